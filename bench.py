@@ -1,0 +1,269 @@
+#!/usr/bin/env python3
+"""Benchmark of the frozen quantized-linear hot path on one MI355X.
+
+Workload (BASELINE.json configs[1], "decode dequant-GEMV"): K=4096, N=14336 (Llama-3-8B FFN
+up-projection), weights ~ N(0, 0.02) quantised once to int8 (per-channel scales) and once to
+int4 (group 128), activations bf16 ~ N(0,1), forward only.  One "step" = one int4 M=1 GEMV
+plus one int8 M=1 GEMV.  Inputs are resident in HBM before the timed region; successive steps
+rotate through >= 512 MB of distinct weight copies so the 256 MB Infinity Cache cannot serve
+the reads.  `value` is algorithmic bytes moved per second (weights + scales + X + Y).
+
+The launches of the timed region are captured once into a HIP graph and replayed, so the GPU,
+not the Python launch path, sets the pace; per-kernel durations for the roofline object come
+from HIP events around single-kernel graphs on the same stream.
+
+Also reported in `extra`: M in {4,16} decode rates, the cache-resident M=1 rate, and the
+compute-bound rows (configs[2..4]) in TFLOP/s.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+K_DEC, N_DEC = 4096, 14336
+
+
+def algorithmic_bytes(kind, M, N=N_DEC, K=K_DEC, group=128):
+    """Bytes one launch has to move: packed weights + scales + X (bf16) + Y (fp32)."""
+    if kind == "int4":
+        w = N * K // 2 + (N * K // group) * 2
+    else:
+        w = N * K + N * 4
+    return w + M * K * 2 + M * N * 4
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary rows (M=4/16, GEMM TFLOP/s)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from caif_amd import capi, torch_ops as T
+
+    capi.lib()                                    # fail loudly when the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+
+    # ---------------------------------------------------------------- synthetic weights, quantised on the GPU
+    w = torch.empty(N_DEC, K_DEC, device=dev).normal_(0, 0.02, generator=gen)
+    p4, s4 = T.quantize_int4_per_group(w, 128)
+    q8, s8 = T.quantize_int8(w.reshape(K_DEC, N_DEC), per_channel=True)     # the reference's [in,out] labelling
+    q8 = q8.reshape(-1)
+    del w
+    copies4 = max(2, -(-512 * 2**20 // algorithmic_bytes("int4", 1)))       # >= 512 MB of distinct weights
+    copies8 = max(2, -(-512 * 2**20 // algorithmic_bytes("int8", 1)))
+    W4 = [T.FrozenWeight(p4.clone(), T.W_INT4_GROUP, s4.clone(), N_DEC, K_DEC, 1, 128) for _ in range(copies4)]
+    W8 = [T.FrozenWeight(q8.clone(), T.W_INT8, s8.clone(), N_DEC, K_DEC, N_DEC) for _ in range(copies8)]
+    X = {m: torch.empty(m, K_DEC, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16) for m in (1, 4, 16)}
+    Y = {m: torch.empty(m, N_DEC, device=dev) for m in (1, 4, 16)}
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+
+    def gemv(fw, m):
+        T.qlinear_forward(X[m], fw, T.BF16, T.F32, out=Y[m], workspace=ws)
+
+    def step(i):
+        gemv(W4[i % copies4], 1)
+        gemv(W8[i % copies8], 1)
+
+    def capture(fn, count):
+        """Record fn(0..count-1) into one HIP graph on a side stream (no memsets are recorded)."""
+        g = torch.cuda.CUDAGraph()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            fn(0)
+            torch.cuda.synchronize()
+            with torch.cuda.graph(g, stream=s):
+                for i in range(count):
+                    fn(i)
+        torch.cuda.synchronize()
+        return g
+
+    def time_graph(g, launches, reps=5):
+        """Average milliseconds per launch, HIP events around graph replays (best of reps)."""
+        g.replay()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) / launches)
+        return best
+
+    # ---------------------------------------------------------------- the timed region: K steps
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    graph = capture(step, args.steps)
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    graph.replay()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    step_bytes = algorithmic_bytes("int4", 1) + algorithmic_bytes("int8", 1)
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---------------------------------------------------------------- per-kernel durations (HIP events)
+    L = 64
+    per = {}
+    for kind, Ws, nc in (("int4", W4, copies4), ("int8", W8, copies8)):
+        for m in (1, 4, 16):
+            if m != 1 and args.no_extra:
+                continue
+            g = capture(lambda i, Ws=Ws, nc=nc, m=m: gemv(Ws[i % nc], m), L)
+            ms = time_graph(g, L)
+            per[(kind, m)] = {"us": ms * 1e3, "GBps": algorithmic_bytes(kind, m) / (ms * 1e-3) / 1e9}
+            del g
+    resident = {}
+    for kind, Ws in (("int4", W4), ("int8", W8)):
+        g = capture(lambda i, Ws=Ws: gemv(Ws[0], 1), L)
+        ms = time_graph(g, L)
+        resident[kind] = algorithmic_bytes(kind, 1) / (ms * 1e-3) / 1e9
+        del g
+
+    dom = ("int8", 1)           # the kernel that takes most of a step
+    roofline = {
+        "bound": "hbm",
+        "kernel": "skinny_forward_kernel<bf16,bf16,int8 per-channel> M=1 K=4096 N=14336",
+        "achieved": round(per[dom]["GBps"], 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(per[dom]["GBps"] / HBM_PEAK_GBS, 4),
+        "avg_launch_us": round(per[dom]["us"], 3),
+        "algorithmic_bytes_per_launch": algorithmic_bytes("int8", 1),
+        "traffic": None,
+    }
+
+    extra = {
+        "decode_GBps": {f"{k}_M{m}": round(v["GBps"], 1) for (k, m), v in per.items()},
+        "decode_us": {f"{k}_M{m}": round(v["us"], 3) for (k, m), v in per.items()},
+        "decode_cache_resident_GBps_M1": {k: round(v, 1) for k, v in resident.items()},
+        "decode_frac_of_hbm_peak_M1": {k: round(per[(k, 1)]["GBps"] / HBM_PEAK_GBS, 4) for k in ("int4", "int8")},
+        "weight_copies_rotated": {"int4": copies4, "int8": copies8},
+    }
+    if not args.no_extra:
+        try:
+            extra.update(compute_bound_rows(torch, T, dev, gen, capture, time_graph))
+        except Exception as e:   # secondary rows must not take the headline down
+            extra["compute_bound_error"] = repr(e)
+
+    out = {
+        "metric": "dequant-GEMM HBM GB/s (M=1 int4/int8) + MFMA TFLOP/s (M=2048 fwd+dX)",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "decode dequant-GEMV K=4096 N=14336 M=1: one int4(g128) + one int8(per-channel) "
+                               "launch per step, weights rotated over >=512 MB (BASELINE configs[1])",
+                   "bytes_per_step": step_bytes},
+        "roofline": roofline,
+        "extra": extra,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(np, q8.cpu().numpy(), s8.cpu().numpy(), p4.cpu().numpy(),
+                                           s4.cpu().view(torch.int16).numpy().view(np.uint16),
+                                           X[1].float().cpu().numpy())
+    print(json.dumps(out))
+
+
+def compute_bound_rows(torch, T, dev, gen, capture, time_graph):
+    """configs[2] and configs[3]: int4 g128 dequant-GEMM forward (+ dX) in TFLOP/s."""
+    rows = {}
+    L = 8
+    for (M, N, K, with_dx) in ((2048, 4096, 4096, True), (2048, 11008, 4096, True), (4096, 11008, 4096, True)):
+        w = torch.empty(N, K, device=dev).normal_(0, 0.02, generator=gen)
+        p, s = T.quantize_int4_per_group(w, 128)
+        del w
+        fw = T.FrozenWeight(p, T.W_INT4_GROUP, s, N, K, 1, 128)
+        x = torch.empty(M, K, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16)
+        dy = torch.empty(M, N, device=dev).normal_(0, 1e-3, generator=gen).to(torch.bfloat16)
+        y = torch.empty(M, N, device=dev)
+        dx = torch.empty(M, K, device=dev)
+        from caif_amd import capi
+        nb = max(capi.lib().caifx_qlinear_workspace_bytes(M, N, K, T.BF16, T.BF16, T.W_INT4_GROUP, b) for b in (0, 1))
+        ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=dev)
+        flops = 2.0 * M * N * K
+        g = capture(lambda i: T.qlinear_forward(x, fw, T.BF16, T.F32, out=y, workspace=ws), L)
+        ms_f = time_graph(g, L, reps=3)
+        del g
+        key = f"int4_M{M}_N{N}_K{K}"
+        rows[key] = {"fwd_us": round(ms_f * 1e3, 2), "fwd_TFLOPs": round(flops / (ms_f * 1e-3) / 1e12, 1)}
+        if with_dx:
+            g = capture(lambda i: T.qlinear_backward_input(dy, fw, T.BF16, T.F32, out=dx, workspace=ws), L)
+            ms_b = time_graph(g, L, reps=3)
+            del g
+            rows[key].update({"dx_us": round(ms_b * 1e3, 2), "dx_TFLOPs": round(flops / (ms_b * 1e-3) / 1e12, 1),
+                              "fwd_dx_frac_of_mfma_peak":
+                                  round(2 * flops / ((ms_f + ms_b) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+    return {"prefill_gemm": rows}
+
+
+def cpu_baseline(np, q8, s8, p4, s4_bits, x_values):
+    """The reference's Host_e path for this layer is cblas_sgemm on an fp32 weight
+    (src/caif_ops_host.cpp:112-139); it has no host dequantiser, so the timed CPU job is the
+    oracle's OpenMP dequantise-to-fp32 followed by that sgemm (numpy's bundled OpenBLAS), on the
+    same M=1 workload.  Bounded: at most ~20 s of CPU work."""
+    from oracle import oracle as orc
+    orc.build()
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    x = np.ascontiguousarray(x_values, np.float32)
+    reps, t_deq, t_gemm = 0, 0.0, 0.0
+    t_start = time.perf_counter()
+    while reps < 20 and time.perf_counter() - t_start < 15.0:
+        t0 = time.perf_counter()
+        w4 = orc.frozen_weight_compute(p4, orc.W_INT4_GROUP, s4_bits, N_DEC, K_DEC, 1, 128, orc.F32)
+        w8 = orc.frozen_weight_compute(q8, orc.W_INT8, s8, N_DEC, K_DEC, N_DEC, 128, orc.F32)
+        t1 = time.perf_counter()
+        y4 = x @ w4.T                              # cblas_sgemm(NoTrans, Trans, M, N, K)
+        y8 = x @ w8.T
+        t2 = time.perf_counter()
+        t_deq += t1 - t0
+        t_gemm += t2 - t1
+        reps += 1
+    del y4, y8
+    step_bytes = algorithmic_bytes("int4", 1) + algorithmic_bytes("int8", 1)
+    per_step = (t_deq + t_gemm) / reps
+    return {
+        "value": round(step_bytes / per_step / 1e9, 3),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{reps} full steps of the same M=1 workload (int4 + int8, K=4096, N=14336): oracle OpenMP "
+                  f"dequantise-to-fp32 ({t_deq / reps * 1e3:.1f} ms/step) + numpy/OpenBLAS sgemm "
+                  f"({t_gemm / reps * 1e3:.1f} ms/step)",
+        "ms_per_step": round(per_step * 1e3, 3),
+    }
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,197 @@
+// extern "C" entry points of the dequant-GEMM seam: argument validation and kernel choice.
+#include "caifx_internal.hpp"
+
+using namespace caifx;
+
+namespace {
+
+int validate_weight(int64_t N, int64_t K, int w_kind, const void *scales, int64_t scale_period, int group_size)
+{
+  (void)N;
+  (void)K;
+  if (w_kind == CAIFX_W_INT4_GROUP) {
+    if (group_size <= 0 || !scales) return CAIFX_ERR_INVALID_ARGUMENT;
+    if (!aligned_to(scales, 2)) return CAIFX_ERR_MISALIGNED;
+  } else if (w_kind == CAIFX_W_INT8) {
+    if (scales) {
+      if (scale_period <= 0) return CAIFX_ERR_INVALID_ARGUMENT;
+      if (!aligned_to(scales, 4)) return CAIFX_ERR_MISALIGNED;
+    }
+  } else {
+    return CAIFX_ERR_INVALID_ARGUMENT;
+  }
+  return CAIFX_OK;
+}
+
+int validate_common(int64_t M, int64_t N, int64_t K, const void *x, int x_dtype, int compute_dtype, void *y,
+                    int y_dtype)
+{
+  if (M < 0 || N <= 0 || K <= 0) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (!valid_dtype(x_dtype) || !valid_dtype(compute_dtype) || !valid_dtype(y_dtype)) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (M > 0 && (!x || !y)) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(x, dtype_size(x_dtype)) || !aligned_to(y, dtype_size(y_dtype))) return CAIFX_ERR_MISALIGNED;
+  return CAIFX_OK;
+}
+
+GemmArgs make_args(int64_t M, int64_t N, int64_t K, const void *x, int x_dtype, int compute_dtype, const void *wq,
+                   int w_kind, const void *scales, int64_t scale_period, int group_size, void *y, int y_dtype,
+                   void *workspace, size_t workspace_bytes)
+{
+  GemmArgs a{};
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.x = x;
+  a.y = y;
+  a.x_dtype = x_dtype;
+  a.y_dtype = y_dtype;
+  a.compute_dtype = compute_dtype;
+  a.w.q = wq;
+  a.w.scales = scales;
+  a.w.kind = w_kind;
+  a.w.group_size = group_size;
+  a.w.scale_period = (w_kind == CAIFX_W_INT8 && scales) ? scale_period : 1;
+  a.workspace = workspace;
+  a.workspace_bytes = workspace_bytes;
+  return a;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *caifx_status_string(int status)
+{
+  switch (status) {
+    case CAIFX_OK: return "ok";
+    case CAIFX_ERR_INVALID_ARGUMENT: return "invalid argument";
+    case CAIFX_ERR_UNSUPPORTED: return "unsupported combination";
+    case CAIFX_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
+    case CAIFX_ERR_LAUNCH_FAILED: return "kernel launch failed";
+    case CAIFX_ERR_MISALIGNED: return "misaligned pointer";
+    default: return "unknown status";
+  }
+}
+
+int caifx_version(void) { return 1000; }
+
+size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtype, int compute_dtype, int w_kind,
+                                     int backward)
+{
+  GemmArgs a{};
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.x_dtype = x_dtype;
+  a.compute_dtype = compute_dtype;
+  a.w.kind = w_kind;
+  return mfma_workspace_bytes(a, backward != 0);
+}
+
+int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K, const void *x, int x_dtype, int compute_dtype,
+                          const void *wq, int w_kind, const void *scales, int64_t scale_period, int group_size,
+                          void *y, int y_dtype, void *workspace, size_t workspace_bytes, caifx_stream_t stream)
+{
+  int st = validate_common(M, N, K, x, x_dtype, compute_dtype, y, y_dtype);
+  if (st != CAIFX_OK) return st;
+  if (!wq) return CAIFX_ERR_INVALID_ARGUMENT;
+  st = validate_weight(N, K, w_kind, scales, scale_period, group_size);
+  if (st != CAIFX_OK) return st;
+  if (M == 0) return CAIFX_OK;
+  const GemmArgs a = make_args(M, N, K, x, x_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, y,
+                               y_dtype, workspace, workspace_bytes);
+  hipStream_t s = as_stream(stream);
+  if (M <= 16) {
+    st = skinny_forward(a, s);
+    if (st != CAIFX_ERR_UNSUPPORTED) return st;
+  }
+  st = mfma_forward(a, s);
+  if (st != CAIFX_ERR_UNSUPPORTED) return st;
+  return generic_forward(a, s);
+}
+
+int caifx_qlinear_backward_input(int64_t M, int64_t N, int64_t K, const void *dy, int dy_dtype, int compute_dtype,
+                                 const void *wq, int w_kind, const void *scales, int64_t scale_period,
+                                 int group_size, void *dx, int dx_dtype, void *workspace, size_t workspace_bytes,
+                                 caifx_stream_t stream)
+{
+  int st = validate_common(M, N, K, dy, dy_dtype, compute_dtype, dx, dx_dtype);
+  if (st != CAIFX_OK) return st;
+  if (!wq) return CAIFX_ERR_INVALID_ARGUMENT;
+  st = validate_weight(N, K, w_kind, scales, scale_period, group_size);
+  if (st != CAIFX_OK) return st;
+  if (M == 0) return CAIFX_OK;
+  const GemmArgs a = make_args(M, N, K, dy, dy_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size,
+                               dx, dx_dtype, workspace, workspace_bytes);
+  hipStream_t s = as_stream(stream);
+  st = mfma_backward(a, s);
+  if (st != CAIFX_ERR_UNSUPPORTED) return st;
+  return generic_backward(a, s);
+}
+
+size_t caifx_qlinear_grouped_workspace_bytes(int num_experts, int64_t total_rows, int64_t N, int64_t K, int x_dtype,
+                                             int compute_dtype, int w_kind, int backward)
+{
+  GemmArgs a{};
+  a.M = total_rows;
+  a.N = N;
+  a.K = K;
+  a.x_dtype = x_dtype;
+  a.compute_dtype = compute_dtype;
+  a.w.kind = w_kind;
+  a.num_experts = num_experts;
+  a.offsets = reinterpret_cast<const int32_t *>(uintptr_t{1});   // marks the grouped form for the size query
+  return mfma_workspace_bytes(a, backward != 0);
+}
+
+static int grouped(bool backward, int num_experts, const int32_t *offsets, int64_t total_rows, int64_t N, int64_t K,
+                   const void *x, int x_dtype, int compute_dtype, const void *const *wq_ptrs, int w_kind,
+                   const void *const *scales_ptrs, int64_t scale_period, int group_size, void *y, int y_dtype,
+                   void *workspace, size_t workspace_bytes, caifx_stream_t stream)
+{
+  int st = validate_common(total_rows, N, K, x, x_dtype, compute_dtype, y, y_dtype);
+  if (st != CAIFX_OK) return st;
+  if (num_experts < 0) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (num_experts == 0 || total_rows == 0) return CAIFX_OK;
+  if (!offsets || !wq_ptrs) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (w_kind == CAIFX_W_INT4_GROUP) {
+    if (group_size <= 0 || !scales_ptrs) return CAIFX_ERR_INVALID_ARGUMENT;
+  } else if (w_kind == CAIFX_W_INT8) {
+    if (scales_ptrs && scale_period <= 0) return CAIFX_ERR_INVALID_ARGUMENT;
+  } else {
+    return CAIFX_ERR_INVALID_ARGUMENT;
+  }
+  GemmArgs a = make_args(total_rows, N, K, x, x_dtype, compute_dtype, nullptr, w_kind, nullptr, scale_period,
+                         group_size, y, y_dtype, workspace, workspace_bytes);
+  a.w.scale_period = (w_kind == CAIFX_W_INT8 && scales_ptrs) ? scale_period : 1;
+  a.offsets = offsets;
+  a.wq_ptrs = wq_ptrs;
+  a.scales_ptrs = scales_ptrs;
+  a.num_experts = num_experts;
+  hipStream_t s = as_stream(stream);
+  st = backward ? mfma_backward(a, s) : mfma_forward(a, s);
+  if (st != CAIFX_ERR_UNSUPPORTED) return st;
+  return backward ? generic_backward(a, s) : generic_forward(a, s);
+}
+
+int caifx_qlinear_grouped_forward(int num_experts, const int32_t *offsets, int64_t total_rows, int64_t N, int64_t K,
+                                  const void *x, int x_dtype, int compute_dtype, const void *const *wq_ptrs,
+                                  int w_kind, const void *const *scales_ptrs, int64_t scale_period, int group_size,
+                                  void *y, int y_dtype, void *workspace, size_t workspace_bytes,
+                                  caifx_stream_t stream)
+{
+  return grouped(false, num_experts, offsets, total_rows, N, K, x, x_dtype, compute_dtype, wq_ptrs, w_kind,
+                 scales_ptrs, scale_period, group_size, y, y_dtype, workspace, workspace_bytes, stream);
+}
+
+int caifx_qlinear_grouped_backward_input(int num_experts, const int32_t *offsets, int64_t total_rows, int64_t N,
+                                         int64_t K, const void *dy, int dy_dtype, int compute_dtype,
+                                         const void *const *wq_ptrs, int w_kind, const void *const *scales_ptrs,
+                                         int64_t scale_period, int group_size, void *dx, int dx_dtype,
+                                         void *workspace, size_t workspace_bytes, caifx_stream_t stream)
+{
+  return grouped(true, num_experts, offsets, total_rows, N, K, dy, dy_dtype, compute_dtype, wq_ptrs, w_kind,
+                 scales_ptrs, scale_period, group_size, dx, dx_dtype, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,98 @@
+// Shared device helpers for the gfx950 frozen quantized-linear kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "caifx.h"
+
+namespace caifx {
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
+
+constexpr int kWave = 64;
+
+inline hipStream_t as_stream(caifx_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline int launch_status()
+{
+  return hipGetLastError() == hipSuccess ? CAIFX_OK : CAIFX_ERR_LAUNCH_FAILED;
+}
+
+inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+template <typename T> struct dtype_code;
+template <> struct dtype_code<float> { static constexpr int value = CAIFX_F32; };
+template <> struct dtype_code<f16_t> { static constexpr int value = CAIFX_F16; };
+template <> struct dtype_code<bf16_t> { static constexpr int value = CAIFX_BF16; };
+
+inline size_t dtype_size(int dt) { return dt == CAIFX_F32 ? 4 : 2; }
+inline bool valid_dtype(int dt) { return dt == CAIFX_F32 || dt == CAIFX_F16 || dt == CAIFX_BF16; }
+
+// fp32 -> T with round-to-nearest-even (v_cvt_pk_bf16_f32 / v_cvt_f16_f32), T -> fp32 exact.
+template <typename T> __device__ __forceinline__ T from_f32(float v) { return static_cast<T>(v); }
+template <typename T> __device__ __forceinline__ float to_f32(T v) { return static_cast<float>(v); }
+// the value an fp32 number has after a cast to T and back
+template <typename T> __device__ __forceinline__ float round_through(float v) { return to_f32<T>(from_f32<T>(v)); }
+template <> __device__ __forceinline__ float round_through<float>(float v) { return v; }
+
+// Byte k of a dword as fp32 (v_cvt_f32_ubyteK: one VALU op, no shift/mask).
+__device__ __forceinline__ float ubyte0_f32(uint32_t v) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(v)); return r; }
+__device__ __forceinline__ float ubyte1_f32(uint32_t v) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(v)); return r; }
+__device__ __forceinline__ float ubyte2_f32(uint32_t v) { float r; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(v)); return r; }
+__device__ __forceinline__ float ubyte3_f32(uint32_t v) { float r; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(v)); return r; }
+
+// Sign-extended nibble `i` (0 = low) of a byte-sized field, as the reference's dequantiser
+// decodes it: code 0x8 is -8.
+__device__ __forceinline__ int nibble_s4(uint32_t byte, int i)
+{
+  return (static_cast<int>(byte << (28 - 4 * i))) >> 28;
+}
+
+// Eight int4 codes of one dword, flat order (nibble j = element j), times one scale.
+// (code * scale) is formed as fma(code + 8, scale, -8*scale): -8*scale is exact and the fused
+// multiply-add rounds the exact product once, so each value equals the reference's
+// float(code) * scale (the sign of a zero aside).  s must be finite.
+__device__ __forceinline__ void dequant_int4x8(uint32_t p, float s, float (&e)[8])
+{
+  const float m8 = -8.0f * s;
+  p ^= 0x88888888u;                       // two's complement nibble -> offset binary (code + 8)
+  const uint32_t lo = p & 0x0F0F0F0Fu;    // elements 0,2,4,6 in bytes 0..3
+  const uint32_t hi = (p >> 4) & 0x0F0F0F0Fu;  // elements 1,3,5,7
+  e[0] = __builtin_fmaf(ubyte0_f32(lo), s, m8);
+  e[1] = __builtin_fmaf(ubyte0_f32(hi), s, m8);
+  e[2] = __builtin_fmaf(ubyte1_f32(lo), s, m8);
+  e[3] = __builtin_fmaf(ubyte1_f32(hi), s, m8);
+  e[4] = __builtin_fmaf(ubyte2_f32(lo), s, m8);
+  e[5] = __builtin_fmaf(ubyte2_f32(hi), s, m8);
+  e[6] = __builtin_fmaf(ubyte3_f32(lo), s, m8);
+  e[7] = __builtin_fmaf(ubyte3_f32(hi), s, m8);
+}
+
+// Four int8 codes of one dword as fp32.
+__device__ __forceinline__ void int8x4_to_f32(uint32_t p, float (&e)[4])
+{
+  e[0] = static_cast<float>(static_cast<int8_t>(p));
+  e[1] = static_cast<float>(static_cast<int8_t>(p >> 8));
+  e[2] = static_cast<float>(static_cast<int8_t>(p >> 16));
+  e[3] = static_cast<float>(static_cast<int>(p) >> 24);
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+}  // namespace caifx

@@ -1,0 +1,46 @@
+// Argument blocks and entry points shared by the dequant-GEMM translation units.
+#pragma once
+
+#include "caifx_common.hpp"
+
+namespace caifx {
+
+// One frozen weight as stored: codes + scales + how a scale is found for flat index f.
+struct QWeight {
+  const void *q;          // int8[N*K] or packed int4[(N*K+1)/2]
+  const void *scales;     // int8: fp32[scale_period] or null; int4: fp16[ceil(N*K/group_size)]
+  int kind;               // caifx_weight_kind
+  int group_size;         // int4 only
+  int64_t scale_period;   // int8 only: scale index = f % scale_period
+};
+
+// One dequant-GEMM problem.  Forward: x [M,K], y [M,N].  Backward: x = dY [M,N], y = dX [M,K].
+// Grouped: offsets != null, rows of expert e are [offsets[e], offsets[e+1]), weight pointers
+// come from wq_ptrs/scales_ptrs, and M is an upper bound on rows.
+struct GemmArgs {
+  int64_t M, N, K;
+  const void *x;
+  void *y;
+  int x_dtype, y_dtype, compute_dtype;
+  QWeight w;
+  const int32_t *offsets;
+  const void *const *wq_ptrs;
+  const void *const *scales_ptrs;
+  int num_experts;
+  void *workspace;
+  size_t workspace_bytes;
+};
+
+int generic_forward(const GemmArgs &a, hipStream_t s);
+int generic_backward(const GemmArgs &a, hipStream_t s);
+
+// M <= 16 decode path (memory bound).  Returns CAIFX_ERR_UNSUPPORTED when the shape is outside
+// its tiling assumptions so that the caller can fall back.
+int skinny_forward(const GemmArgs &a, hipStream_t s);
+
+// Large-M MFMA path (compute bound), forward and input gradient, plain and grouped.
+int mfma_forward(const GemmArgs &a, hipStream_t s);
+int mfma_backward(const GemmArgs &a, hipStream_t s);
+size_t mfma_workspace_bytes(const GemmArgs &a, bool backward);
+
+}  // namespace caifx

@@ -1,0 +1,379 @@
+// Quantise / dequantise / cast kernels for gfx950.
+//
+// Numerics contract (what makes codes and scales bit-identical to the reference's
+// src/caif_cuda_kernels_quant.cu): IEEE binary32 division for max/127, max/7 and 1/scale,
+// a single rounding for x * inv_scale, clamp before round, round-half-to-even (v_rndne_f32),
+// fp32 -> fp16 scale by round-half-to-even (v_cvt_f16_f32), int4 codes from the UNROUNDED
+// fp32 scale.  Max reductions are order independent, so parallelising them changes nothing.
+// No multiply feeds an add in these kernels; contraction is switched off anyway.
+#include "caifx_common.hpp"
+
+#pragma clang fp contract(off)
+
+namespace caifx {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr float kInt8Max = 127.0f;
+constexpr float kInt4Max = 7.0f;
+
+inline int grid_for(int64_t work_items, int block = kBlock)
+{
+  return static_cast<int>((work_items + block - 1) / block);
+}
+
+__device__ __forceinline__ float clamp_sym(float v, float limit)
+{
+  if (v > limit) v = limit;
+  else if (v < -limit) v = -limit;
+  return v;
+}
+
+// ------------------------------------------------------------------ casts
+template <typename In, typename Out>
+__global__ void cast_kernel(const In *__restrict__ in, Out *__restrict__ out, int64_t n)
+{
+  int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+  if (i + 4 <= n) {
+    In v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = in[i + j];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[i + j] = static_cast<Out>(static_cast<float>(v[j]));
+  } else {
+    for (; i < n; ++i) out[i] = static_cast<Out>(static_cast<float>(in[i]));
+  }
+}
+
+__global__ void cast_f32_to_int8_kernel(const float *__restrict__ in, int8_t *__restrict__ out, int64_t n)
+{
+  int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+  int64_t end = i + 4 < n ? i + 4 : n;
+  for (; i < end; ++i) out[i] = static_cast<int8_t>(rintf(clamp_sym(in[i], kInt8Max)));
+}
+
+template <typename In, typename Out>
+int launch_cast(const In *in, Out *out, int64_t n, hipStream_t s)
+{
+  if (n <= 0) return CAIFX_OK;
+  if (!in || !out) return CAIFX_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL((cast_kernel<In, Out>), dim3(grid_for((n + 3) / 4)), dim3(kBlock), 0, s, in, out, n);
+  return launch_status();
+}
+
+// ------------------------------------------------------------------ absmax reductions
+__global__ void fill_u32_kernel(uint32_t *p, int64_t n, uint32_t v)
+{
+  int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// max |x| over the whole tensor -> atomicMax on the bit pattern (non-negative floats order
+// like unsigned integers).  `v > m` drops NaNs exactly like the reference's comparison.
+__global__ void absmax_tensor_kernel(const float *__restrict__ in, uint32_t *__restrict__ acc, int64_t n)
+{
+  __shared__ float part[kBlock / kWave];
+  float m = 0.0f;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
+    float v = fabsf(in[i]);
+    if (v > m) m = v;
+  }
+  m = wave_max(m);
+  if ((threadIdx.x & (kWave - 1)) == 0) part[threadIdx.x / kWave] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kBlock / kWave; ++w) m = fmaxf(m, part[w]);
+    if (m > 0.0f) atomicMax(acc, __float_as_uint(m));
+  }
+}
+
+// max over rows of |x[r, c]| for a [rows, cols] row-major tensor; one thread per column and
+// a chunk of rows, coalesced across the columns of a block.
+constexpr int kRowChunk = 64;
+__global__ void absmax_columns_kernel(const float *__restrict__ in, uint32_t *__restrict__ acc, int rows, int cols)
+{
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= cols) return;
+  const int r0 = blockIdx.y * kRowChunk;
+  const int r1 = r0 + kRowChunk < rows ? r0 + kRowChunk : rows;
+  float m = 0.0f;
+  for (int r = r0; r < r1; ++r) {
+    float v = fabsf(in[static_cast<int64_t>(r) * cols + c]);
+    if (v > m) m = v;
+  }
+  if (m > 0.0f) atomicMax(acc + c, __float_as_uint(m));
+}
+
+// in place: max|x| -> scale = max / 127 (1.0 when max is zero)
+__global__ void finalize_int8_scale_kernel(float *scales, int count)
+{
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= count) return;
+  const float m = scales[c];
+  scales[c] = (m > 0.0f) ? m / kInt8Max : 1.0f;
+}
+
+// q = rint(clamp(x * (1/scale[f % period], +-127)); four consecutive elements per thread
+__global__ void quantize_int8_kernel(const float *__restrict__ in, int8_t *__restrict__ out,
+                                     const float *__restrict__ scales, int64_t n, int period)
+{
+  int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+  if (i >= n) return;
+  int col = static_cast<int>(i % period);
+  const int cnt = (n - i) < 4 ? static_cast<int>(n - i) : 4;
+  for (int j = 0; j < cnt; ++j) {
+    const float s = scales[col];
+    const float inv_s = (s > 0.0f) ? 1.0f / s : 0.0f;
+    out[i + j] = static_cast<int8_t>(rintf(clamp_sym(in[i + j] * inv_s, kInt8Max)));
+    if (++col == period) col = 0;
+  }
+}
+
+__global__ void dequantize_int8_kernel(const int8_t *__restrict__ in, float *__restrict__ out,
+                                       const float *__restrict__ scales, int64_t n, int period)
+{
+  int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+  if (i >= n) return;
+  int col = static_cast<int>(i % period);
+  const int cnt = (n - i) < 4 ? static_cast<int>(n - i) : 4;
+  for (int j = 0; j < cnt; ++j) {
+    out[i + j] = static_cast<float>(in[i + j]) * scales[col];
+    if (++col == period) col = 0;
+  }
+}
+
+// ------------------------------------------------------------------ int4 per-group
+// Fast path: each thread owns 8 consecutive elements (one dword of packed output); a team of
+// group_size/8 adjacent lanes owns one group and shares its max through wave shuffles.
+// Needs group_size % 8 == 0 and group_size/8 a power of two <= 64.
+__global__ void quantize_int4_team_kernel(const float *__restrict__ in, uint8_t *__restrict__ packed,
+                                          f16_t *__restrict__ scales, int64_t n, int group_size, int team)
+{
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t base = gid * 8;
+  float x[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) x[j] = (base + j < n) ? in[base + j] : 0.0f;
+  float m = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    float a = fabsf(x[j]);
+    if (a > m) m = a;
+  }
+  for (int o = team >> 1; o > 0; o >>= 1) {
+    float other = __shfl_xor(m, o, 64);
+    if (other > m) m = other;
+  }
+  if (base >= n) return;
+  const float scale = (m == 0.0f) ? 0.0f : m / kInt4Max;
+  if ((gid & (team - 1)) == 0) scales[base / group_size] = static_cast<f16_t>(scale);
+  const float inv = (scale == 0.0f) ? 0.0f : 1.0f / scale;
+  uint32_t word = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    int q = static_cast<int>(rintf(clamp_sym(x[j] * inv, kInt4Max))) & 0xF;
+    if (base + j >= n) q = 0;
+    word |= static_cast<uint32_t>(q) << (4 * j);
+  }
+  const int64_t byte0 = base / 2;
+  const int64_t nbytes = (n + 1) / 2;
+  if (byte0 + 4 <= nbytes) {
+    *reinterpret_cast<uint32_t *>(packed + byte0) = word;
+  } else {
+    for (int64_t b = byte0; b < nbytes; ++b) packed[b] = static_cast<uint8_t>(word >> (8 * (b - byte0)));
+  }
+}
+
+// Any (even) group size: one thread per group, serial over the group.
+__global__ void quantize_int4_serial_kernel(const float *__restrict__ in, uint8_t *__restrict__ packed,
+                                            f16_t *__restrict__ scales, int64_t n, int group_size)
+{
+  const int64_t g = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t num_groups = (n + group_size - 1) / group_size;
+  if (g >= num_groups) return;
+  const int64_t start = g * group_size;
+  const int64_t end = start + group_size < n ? start + group_size : n;
+  float m = 0.0f;
+  for (int64_t i = start; i < end; ++i) {
+    float a = fabsf(in[i]);
+    if (a > m) m = a;
+  }
+  const float scale = (m == 0.0f) ? 0.0f : m / kInt4Max;
+  scales[g] = static_cast<f16_t>(scale);
+  const float inv = (scale == 0.0f) ? 0.0f : 1.0f / scale;
+  for (int64_t i = start; i < end; i += 2) {
+    int q0 = static_cast<int>(rintf(clamp_sym(in[i] * inv, kInt4Max))) & 0xF;
+    int q1 = 0;
+    if (i + 1 < end) q1 = static_cast<int>(rintf(clamp_sym(in[i + 1] * inv, kInt4Max))) & 0xF;
+    packed[i / 2] = static_cast<uint8_t>(q0 | (q1 << 4));
+  }
+}
+
+// out[f] = float(code) * float(scale[f / group]); 8 elements (one packed dword) per thread
+__global__ void dequantize_int4_x8_kernel(const uint8_t *__restrict__ packed, const f16_t *__restrict__ scales,
+                                          float *__restrict__ out, int64_t n, int group_size)
+{
+  const int64_t base = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 8;
+  if (base >= n) return;
+  if (base + 8 <= n) {
+    const uint32_t w = *reinterpret_cast<const uint32_t *>(packed + base / 2);
+    const float s = static_cast<float>(scales[base / group_size]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out[base + j] = static_cast<float>(nibble_s4(w >> (4 * j), 0)) * s;
+  } else {
+    for (int64_t f = base; f < n; ++f) {
+      const uint32_t b = packed[f / 2];
+      out[f] = static_cast<float>(nibble_s4(b, static_cast<int>(f & 1))) * static_cast<float>(scales[f / group_size]);
+    }
+  }
+}
+
+__global__ void dequantize_int4_scalar_kernel(const uint8_t *__restrict__ packed, const f16_t *__restrict__ scales,
+                                              float *__restrict__ out, int64_t n, int group_size)
+{
+  const int64_t f = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (f >= n) return;
+  const uint32_t b = packed[f / 2];
+  out[f] = static_cast<float>(nibble_s4(b, static_cast<int>(f & 1))) * static_cast<float>(scales[f / group_size]);
+}
+
+}  // namespace
+}  // namespace caifx
+
+using namespace caifx;
+
+extern "C" {
+
+int caifx_convert_fp32_to_fp16(const float *input, void *output, int64_t n, caifx_stream_t stream)
+{
+  return launch_cast<float, f16_t>(input, static_cast<f16_t *>(output), n, as_stream(stream));
+}
+int caifx_convert_fp16_to_fp32(const void *input, float *output, int64_t n, caifx_stream_t stream)
+{
+  return launch_cast<f16_t, float>(static_cast<const f16_t *>(input), output, n, as_stream(stream));
+}
+int caifx_convert_fp32_to_bf16(const float *input, void *output, int64_t n, caifx_stream_t stream)
+{
+  return launch_cast<float, bf16_t>(input, static_cast<bf16_t *>(output), n, as_stream(stream));
+}
+int caifx_convert_bf16_to_fp32(const void *input, float *output, int64_t n, caifx_stream_t stream)
+{
+  return launch_cast<bf16_t, float>(static_cast<const bf16_t *>(input), output, n, as_stream(stream));
+}
+int caifx_convert_fp32_to_int8(const float *input, void *output, int64_t n, caifx_stream_t stream)
+{
+  if (n <= 0) return CAIFX_OK;
+  if (!input || !output) return CAIFX_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(cast_f32_to_int8_kernel, dim3(grid_for((n + 3) / 4)), dim3(kBlock), 0, as_stream(stream),
+                     input, static_cast<int8_t *>(output), n);
+  return launch_status();
+}
+int caifx_convert_int8_to_fp32(const void *input, float *output, int64_t n, caifx_stream_t stream)
+{
+  return launch_cast<int8_t, float>(static_cast<const int8_t *>(input), output, n, as_stream(stream));
+}
+
+int caifx_quantize_int8_per_tensor(const float *input, void *output, void *scale, int64_t n,
+                                   caifx_stream_t stream)
+{
+  if (n <= 0) return CAIFX_OK;
+  if (!input || !output || !scale) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(input, 4) || !aligned_to(scale, 4)) return CAIFX_ERR_MISALIGNED;
+  hipStream_t s = as_stream(stream);
+  // a fill kernel, not hipMemsetAsync: safe to record into a captured graph
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, s, static_cast<uint32_t *>(scale), int64_t{1}, 0u);
+  int blocks = grid_for(n);
+  if (blocks > 2048) blocks = 2048;
+  hipLaunchKernelGGL(absmax_tensor_kernel, dim3(blocks), dim3(kBlock), 0, s, input, static_cast<uint32_t *>(scale), n);
+  hipLaunchKernelGGL(finalize_int8_scale_kernel, dim3(1), dim3(64), 0, s, static_cast<float *>(scale), 1);
+  hipLaunchKernelGGL(quantize_int8_kernel, dim3(grid_for((n + 3) / 4)), dim3(kBlock), 0, s, input,
+                     static_cast<int8_t *>(output), static_cast<const float *>(scale), n, 1);
+  return launch_status();
+}
+
+int caifx_dequantize_int8_per_tensor(const void *input, float *output, const void *scale, int64_t n,
+                                     caifx_stream_t stream)
+{
+  if (n <= 0) return CAIFX_OK;
+  if (!input || !output || !scale) return CAIFX_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(dequantize_int8_kernel, dim3(grid_for((n + 3) / 4)), dim3(kBlock), 0, as_stream(stream),
+                     static_cast<const int8_t *>(input), output, static_cast<const float *>(scale), n, 1);
+  return launch_status();
+}
+
+int caifx_quantize_int8_per_channel(const float *input, void *output, void *scales, int rows, int cols,
+                                    caifx_stream_t stream)
+{
+  if (rows <= 0 || cols <= 0) return CAIFX_OK;
+  if (!input || !output || !scales) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(input, 4) || !aligned_to(scales, 4)) return CAIFX_ERR_MISALIGNED;
+  hipStream_t s = as_stream(stream);
+  const int64_t n = static_cast<int64_t>(rows) * cols;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(cols)), dim3(kBlock), 0, s, static_cast<uint32_t *>(scales),
+                     static_cast<int64_t>(cols), 0u);
+  hipLaunchKernelGGL(absmax_columns_kernel, dim3(grid_for(cols), (rows + kRowChunk - 1) / kRowChunk), dim3(kBlock), 0, s,
+                     input, static_cast<uint32_t *>(scales), rows, cols);
+  hipLaunchKernelGGL(finalize_int8_scale_kernel, dim3(grid_for(cols)), dim3(kBlock), 0, s,
+                     static_cast<float *>(scales), cols);
+  hipLaunchKernelGGL(quantize_int8_kernel, dim3(grid_for((n + 3) / 4)), dim3(kBlock), 0, s, input,
+                     static_cast<int8_t *>(output), static_cast<const float *>(scales), n, cols);
+  return launch_status();
+}
+
+int caifx_dequantize_int8_per_channel(const void *input, float *output, const void *scales, int rows,
+                                      int cols, caifx_stream_t stream)
+{
+  if (rows <= 0 || cols <= 0) return CAIFX_OK;
+  if (!input || !output || !scales) return CAIFX_ERR_INVALID_ARGUMENT;
+  const int64_t n = static_cast<int64_t>(rows) * cols;
+  hipLaunchKernelGGL(dequantize_int8_kernel, dim3(grid_for((n + 3) / 4)), dim3(kBlock), 0, as_stream(stream),
+                     static_cast<const int8_t *>(input), output, static_cast<const float *>(scales), n, cols);
+  return launch_status();
+}
+
+int caifx_quantize_to_int4(const float *input, void *packed_output, void *scales_output,
+                           int64_t num_elements, int group_size, caifx_stream_t stream)
+{
+  if (num_elements <= 0) return CAIFX_OK;
+  if (!input || !packed_output || !scales_output || group_size <= 0) return CAIFX_ERR_INVALID_ARGUMENT;
+  if ((group_size & 1) && num_elements > group_size) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(input, 4) || !aligned_to(scales_output, 2)) return CAIFX_ERR_MISALIGNED;
+  hipStream_t s = as_stream(stream);
+  const int team = group_size / 8;
+  const bool team_ok = (group_size % 8 == 0) && team >= 1 && team <= 64 && (team & (team - 1)) == 0 &&
+                       aligned_to(packed_output, 4);
+  if (team_ok) {
+    const int64_t threads = (num_elements + 7) / 8;
+    hipLaunchKernelGGL(quantize_int4_team_kernel, dim3(grid_for(threads)), dim3(kBlock), 0, s, input,
+                       static_cast<uint8_t *>(packed_output), static_cast<f16_t *>(scales_output), num_elements,
+                       group_size, team);
+  } else {
+    const int64_t groups = (num_elements + group_size - 1) / group_size;
+    hipLaunchKernelGGL(quantize_int4_serial_kernel, dim3(grid_for(groups)), dim3(kBlock), 0, s, input,
+                       static_cast<uint8_t *>(packed_output), static_cast<f16_t *>(scales_output), num_elements,
+                       group_size);
+  }
+  return launch_status();
+}
+
+int caifx_dequantize_int4(const void *packed_data, const void *scales, float *output,
+                          int64_t num_elements, int group_size, caifx_stream_t stream)
+{
+  if (num_elements <= 0) return CAIFX_OK;
+  if (!packed_data || !scales || !output || group_size <= 0) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(output, 4) || !aligned_to(scales, 2)) return CAIFX_ERR_MISALIGNED;
+  hipStream_t s = as_stream(stream);
+  if (group_size % 8 == 0 && aligned_to(packed_data, 4)) {
+    hipLaunchKernelGGL(dequantize_int4_x8_kernel, dim3(grid_for((num_elements + 7) / 8)), dim3(kBlock), 0, s,
+                       static_cast<const uint8_t *>(packed_data), static_cast<const f16_t *>(scales), output,
+                       num_elements, group_size);
+  } else {
+    hipLaunchKernelGGL(dequantize_int4_scalar_kernel, dim3(grid_for(num_elements)), dim3(kBlock), 0, s,
+                       static_cast<const uint8_t *>(packed_data), static_cast<const f16_t *>(scales), output,
+                       num_elements, group_size);
+  }
+  return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,227 @@
+"""Thin callers of the C ABI for torch-owned device buffers (tests and bench.py plumbing).
+
+torch supplies device memory and the current HIP stream; every computation is a
+call into libcaifx.so.  Function names follow the reference's CAIF_Ops entry
+points (src/caif_ops.cpp:504-680); argument meaning is the same.
+"""
+import torch
+
+from . import capi
+from .capi import F32, F16, BF16, W_INT8, W_INT4_GROUP
+
+TORCH_DTYPE = {F32: torch.float32, F16: torch.float16, BF16: torch.bfloat16}
+CODE_OF = {v: k for k, v in TORCH_DTYPE.items()}
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            # CAIF_Ops quantise entry points throw for Host_e tensors (src/caif_ops.cpp:514-517)
+            raise RuntimeError("host backend not supported")
+        if t is not None and not t.is_contiguous():
+            raise RuntimeError("tensor must be contiguous")
+
+
+# ------------------------------------------------------------------ CAIF_Ops::Quantize* / Dequantize*
+def quantize_int8(x, per_channel):
+    """CAIF_Ops::QuantizeInt8 (src/caif_ops_device.cpp:1517-1573).  Returns (codes, scales)."""
+    _need_cuda(x)
+    if x.dtype != torch.float32:
+        raise RuntimeError("QuantizeInt8: input must be fp32")
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    if not per_channel:
+        s = torch.empty(1, dtype=torch.float32, device=x.device)
+        capi.call("caifx_quantize_int8_per_tensor", _ptr(x), _ptr(q), _ptr(s), x.numel(), _stream())
+        return q, s
+    if x.dim() != 2:
+        raise RuntimeError("QuantizeInt8 PerChannel: input must be 2D")
+    rows, cols = x.shape
+    s = torch.empty(cols, dtype=torch.float32, device=x.device)
+    capi.call("caifx_quantize_int8_per_channel", _ptr(x), _ptr(q), _ptr(s), rows, cols, _stream())
+    return q, s
+
+
+def dequantize_int8(q, scales, per_channel):
+    """CAIF_Ops::DequantizeInt8 (src/caif_ops_device.cpp:1584-1640)."""
+    _need_cuda(q, scales)
+    out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    if not per_channel:
+        if scales.numel() != 1:
+            raise RuntimeError("DequantizeInt8 PerTensor: scales must have 1 element")
+        capi.call("caifx_dequantize_int8_per_tensor", _ptr(q), _ptr(out), _ptr(scales), q.numel(), _stream())
+        return out
+    if q.dim() != 2:
+        raise RuntimeError("DequantizeInt8 PerChannel: input must be 2D")
+    rows, cols = q.shape
+    if scales.numel() != cols:
+        raise RuntimeError("DequantizeInt8 PerChannel: scales length must equal cols")
+    capi.call("caifx_dequantize_int8_per_channel", _ptr(q), _ptr(out), _ptr(scales), rows, cols, _stream())
+    return out
+
+
+def quantize_int4_per_group(x, group_size):
+    """CAIF_Ops::QuantizeInt4PerGroup (src/caif_ops_device.cpp:1651-1687).  Returns (packed, fp16 scales)."""
+    _need_cuda(x)
+    if x.dtype != torch.float32:
+        raise RuntimeError("QuantizeInt4PerGroup: input must be fp32")
+    if group_size == 0:
+        raise RuntimeError("QuantizeInt4PerGroup: group_size must be > 0")
+    n = x.numel()
+    packed = torch.empty((n + 1) // 2, dtype=torch.uint8, device=x.device)
+    scales = torch.empty((n + group_size - 1) // group_size, dtype=torch.float16, device=x.device)
+    capi.call("caifx_quantize_to_int4", _ptr(x), _ptr(packed), _ptr(scales), n, group_size, _stream())
+    return packed, scales
+
+
+def dequantize_int4_per_group(packed, scales, n, group_size):
+    """CAIF_Ops::DequantizeInt4PerGroup (src/caif_ops_device.cpp:1698-1734)."""
+    _need_cuda(packed, scales)
+    if group_size == 0:
+        raise RuntimeError("DequantizeInt4PerGroup: group_size must be > 0")
+    if scales.numel() != (n + group_size - 1) // group_size:
+        raise RuntimeError("DequantizeInt4PerGroup: scales length must equal num_groups")
+    out = torch.empty(n, dtype=torch.float32, device=packed.device)
+    capi.call("caifx_dequantize_int4", _ptr(packed), _ptr(scales), _ptr(out), n, group_size, _stream())
+    return out
+
+
+_CASTS = {
+    (torch.float32, torch.float16): "caifx_convert_fp32_to_fp16",
+    (torch.float16, torch.float32): "caifx_convert_fp16_to_fp32",
+    (torch.float32, torch.bfloat16): "caifx_convert_fp32_to_bf16",
+    (torch.bfloat16, torch.float32): "caifx_convert_bf16_to_fp32",
+    (torch.float32, torch.int8): "caifx_convert_fp32_to_int8",
+    (torch.int8, torch.float32): "caifx_convert_int8_to_fp32",
+}
+
+
+def convert(x, dtype):
+    """The cast kernels behind CAIF_DeviceTensor::To (src/caif_device_tensor.cpp:604-706)."""
+    _need_cuda(x)
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    capi.call(_CASTS[(x.dtype, dtype)], _ptr(x), _ptr(out), x.numel(), _stream())
+    return out
+
+
+# ------------------------------------------------------------------ frozen linear
+class FrozenWeight:
+    """Device storage of one CAIF_DeviceFrozenLinear: codes, scales and the scale scheme."""
+
+    def __init__(self, wq, w_kind, scales, N, K, scale_period=1, group_size=128):
+        self.wq, self.w_kind, self.scales = wq, w_kind, scales
+        self.N, self.K, self.scale_period, self.group_size = N, K, scale_period, group_size
+
+
+def _workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+def qlinear_forward(x, fw, compute_dtype, y_dtype=F32, out=None, workspace=None):
+    """caifx_qlinear_forward on x [..., K]; returns y [M, N]."""
+    _need_cuda(x)
+    M = x.numel() // fw.K
+    y = out if out is not None else torch.empty((M, fw.N), dtype=TORCH_DTYPE[y_dtype], device=x.device)
+    xd = CODE_OF[x.dtype]
+    if workspace is None:
+        workspace = _workspace(capi.lib().caifx_qlinear_workspace_bytes(M, fw.N, fw.K, xd, compute_dtype,
+                                                                       fw.w_kind, 0), x.device)
+    capi.call("caifx_qlinear_forward", M, fw.N, fw.K, _ptr(x), xd, compute_dtype, _ptr(fw.wq), fw.w_kind,
+              _ptr(fw.scales), fw.scale_period, fw.group_size, _ptr(y), y_dtype, _ptr(workspace),
+              workspace.numel(), _stream())
+    return y
+
+
+def qlinear_backward_input(dy, fw, compute_dtype, dx_dtype=F32, out=None, workspace=None):
+    """caifx_qlinear_backward_input on dy [..., N]; returns dx [M, K]."""
+    _need_cuda(dy)
+    M = dy.numel() // fw.N
+    dx = out if out is not None else torch.empty((M, fw.K), dtype=TORCH_DTYPE[dx_dtype], device=dy.device)
+    yd = CODE_OF[dy.dtype]
+    if workspace is None:
+        workspace = _workspace(capi.lib().caifx_qlinear_workspace_bytes(M, fw.N, fw.K, yd, compute_dtype,
+                                                                       fw.w_kind, 1), dy.device)
+    capi.call("caifx_qlinear_backward_input", M, fw.N, fw.K, _ptr(dy), yd, compute_dtype, _ptr(fw.wq),
+              fw.w_kind, _ptr(fw.scales), fw.scale_period, fw.group_size, _ptr(dx), dx_dtype,
+              _ptr(workspace), workspace.numel(), _stream())
+    return dx
+
+
+class GroupedFrozenWeights:
+    """E frozen linears of one shape (one per expert), addressed through device pointer arrays."""
+
+    def __init__(self, weights):
+        w0 = weights[0]
+        self.weights = weights
+        self.N, self.K, self.w_kind = w0.N, w0.K, w0.w_kind
+        self.scale_period, self.group_size = w0.scale_period, w0.group_size
+        dev = w0.wq.device
+        self.wq_ptrs = torch.tensor([w.wq.data_ptr() for w in weights], dtype=torch.int64, device=dev)
+        self.scales_ptrs = None
+        if w0.scales is not None:
+            self.scales_ptrs = torch.tensor([w.scales.data_ptr() for w in weights], dtype=torch.int64, device=dev)
+
+
+def _grouped(name, backward, x, offsets, gw, compute_dtype, out_dtype, out, workspace):
+    _need_cuda(x, offsets)
+    in_dim = gw.N if backward else gw.K
+    out_dim = gw.K if backward else gw.N
+    rows = x.numel() // in_dim
+    y = out if out is not None else torch.zeros((rows, out_dim), dtype=TORCH_DTYPE[out_dtype], device=x.device)
+    xd = CODE_OF[x.dtype]
+    E = len(gw.weights)
+    if workspace is None:
+        workspace = _workspace(capi.lib().caifx_qlinear_grouped_workspace_bytes(
+            E, rows, gw.N, gw.K, xd, compute_dtype, gw.w_kind, int(backward)), x.device)
+    capi.call(name, E, _ptr(offsets), rows, gw.N, gw.K, _ptr(x), xd, compute_dtype, _ptr(gw.wq_ptrs), gw.w_kind,
+              _ptr(gw.scales_ptrs), gw.scale_period, gw.group_size, _ptr(y), out_dtype, _ptr(workspace),
+              workspace.numel(), _stream())
+    return y
+
+
+def qlinear_grouped_forward(x, offsets, gw, compute_dtype, y_dtype=F32, out=None, workspace=None):
+    return _grouped("caifx_qlinear_grouped_forward", False, x, offsets, gw, compute_dtype, y_dtype, out, workspace)
+
+
+def qlinear_grouped_backward_input(dy, offsets, gw, compute_dtype, dx_dtype=F32, out=None, workspace=None):
+    return _grouped("caifx_qlinear_grouped_backward_input", True, dy, offsets, gw, compute_dtype, dx_dtype, out,
+                    workspace)
+
+
+# ------------------------------------------------------------------ element-wise
+def _ew(name, n_in, a, b=None):
+    _need_cuda(a, b)
+    out = torch.empty_like(a)
+    dt = CODE_OF[a.dtype]
+    if n_in == 1:
+        capi.call(name, _ptr(a), _ptr(out), a.numel(), dt, _stream())
+    else:
+        capi.call(name, _ptr(a), _ptr(b), _ptr(out), a.numel(), dt, _stream())
+    return out
+
+
+def silu(x):
+    return _ew("caifx_silu", 1, x)
+
+
+def silu_backward(x, grad_out):
+    return _ew("caifx_silu_backward", 2, x, grad_out)
+
+
+def multiply(a, b):
+    return _ew("caifx_multiply", 2, a, b)
+
+
+def add(a, b):
+    return _ew("caifx_add", 2, a, b)
+
+
+def silu_multiply(gate, up):
+    return _ew("caifx_silu_multiply", 2, gate, up)

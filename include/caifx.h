@@ -1,0 +1,203 @@
+/*
+ * caifx.h -- C ABI of the MI355X (gfx950) frozen quantized-linear kernels.
+ *
+ * This is the seam at which CAIF's C++ host code (CAIF_Ops quantise entry
+ * points, CAIF_DeviceFrozenLinear, CAIF_DeviceMoEFrozenExpert) meets device
+ * code.  Every entry point below replaces either one launcher declared in the
+ * reference's include/caif/caif_cuda_kernels_quant.cuh or one vendor GEMM call
+ * inside the frozen layers; the reference interface it replaces is cited as
+ * file:line relative to the reference checkout (cppaif/caif).
+ *
+ * Conventions
+ *  - Plain C: raw device pointers, element counts (not bytes), enums as int.
+ *  - `stream` is a hipStream_t passed as void*; NULL is the default stream.
+ *    All work is enqueued on it; no entry point synchronises the host, and
+ *    none allocates or frees memory: scratch comes in through `workspace`.
+ *  - Return value: CAIFX_OK (0) or a caifx_status error code.  The reference
+ *    throws CAIF_Exception where these return non-zero; the C++ host layer
+ *    maps a non-zero status back to THROW_CAIFE.
+ *  - Like the reference launchers, an empty problem (n <= 0, rows <= 0, ...)
+ *    is a successful no-op.
+ *  - Weight layout is the reference's, untouched: W is logically [N,K]
+ *    row-major (N = OutputDim, K = InputDim), flat index f = n*K + k
+ *    (src/caif_device_frozen_linear.cpp:345).  int8 holds one code per byte;
+ *    int4 holds two codes per byte, even f in the low nibble, two's complement
+ *    (src/caif_cuda_kernels_quant.cu:205-237).
+ */
+#ifndef CAIFX_H
+#define CAIFX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *caifx_stream_t;            /* hipStream_t */
+
+#if defined(__GNUC__)
+#define CAIFX_API __attribute__((visibility("default")))
+#else
+#define CAIFX_API
+#endif
+
+enum caifx_status {
+  CAIFX_OK = 0,
+  CAIFX_ERR_INVALID_ARGUMENT = 1,        /* null pointer, negative size, bad enum, group_size == 0 ... */
+  CAIFX_ERR_UNSUPPORTED = 2,             /* a combination this build has no kernel for */
+  CAIFX_ERR_WORKSPACE_TOO_SMALL = 3,
+  CAIFX_ERR_LAUNCH_FAILED = 4,           /* hipGetLastError() != hipSuccess after a launch */
+  CAIFX_ERR_MISALIGNED = 5               /* pointer not aligned to its element type */
+};
+
+/* Float element types (CAIF_DataType::Float32 / Float16 / BFloat16). */
+enum caifx_dtype { CAIFX_F32 = 0, CAIFX_F16 = 1, CAIFX_BF16 = 2 };
+
+/* Stored weight kinds of a frozen linear.
+ *  CAIFX_W_INT8:       one int8 code per element; W[n,k] = code * scales[(n*K+k) % scale_period].
+ *                      scale_period 1 is CAIF_Ops::QuantScheme_e::PerTensor_e; scale_period N is
+ *                      what PerChannel_e means once the layer reads the buffer as [N,K]
+ *                      (src/caif_device_frozen_linear.cpp:356-361 with
+ *                      src/caif_cuda_kernels_quant.cu:561-574).  scales == NULL is the
+ *                      "int8 without scales" branch, a plain widening cast (:373-375).
+ *  CAIFX_W_INT4_GROUP: packed nibbles; W[n,k] = code * fp16 scales[(n*K+k) / group_size]
+ *                      (src/caif_cuda_kernels_quant.cu:233-235). */
+enum caifx_weight_kind { CAIFX_W_INT8 = 0, CAIFX_W_INT4_GROUP = 1 };
+
+CAIFX_API const char *caifx_status_string(int status);
+/* ABI version of this header: major*1000 + minor. */
+CAIFX_API int caifx_version(void);
+
+/* ------------------------------------------------------------------------- */
+/* Seam 1: kernel launchers (include/caif/caif_cuda_kernels_quant.cuh)        */
+/* ------------------------------------------------------------------------- */
+
+/* launch_convert_fp32_to_fp16  (caif_cuda_kernels_quant.cuh:47-50)  RNE */
+CAIFX_API int caifx_convert_fp32_to_fp16(const float *input, void *output, int64_t n, caifx_stream_t stream);
+/* launch_convert_fp16_to_fp32  (caif_cuda_kernels_quant.cuh:56-59) */
+CAIFX_API int caifx_convert_fp16_to_fp32(const void *input, float *output, int64_t n, caifx_stream_t stream);
+/* launch_convert_fp32_to_bf16  (caif_cuda_kernels_quant.cuh:68-71)  RNE, NaN stays NaN */
+CAIFX_API int caifx_convert_fp32_to_bf16(const float *input, void *output, int64_t n, caifx_stream_t stream);
+/* launch_convert_bf16_to_fp32  (caif_cuda_kernels_quant.cuh:80-83) */
+CAIFX_API int caifx_convert_bf16_to_fp32(const void *input, float *output, int64_t n, caifx_stream_t stream);
+/* launch_convert_fp32_to_int8  (caif_cuda_kernels_quant.cuh:96-99)  clamp to +-127, then RNE */
+CAIFX_API int caifx_convert_fp32_to_int8(const float *input, void *output, int64_t n, caifx_stream_t stream);
+/* launch_convert_int8_to_fp32  (caif_cuda_kernels_quant.cuh:108-111) */
+CAIFX_API int caifx_convert_int8_to_fp32(const void *input, float *output, int64_t n, caifx_stream_t stream);
+
+/* launch_quantize_int8_per_tensor  (caif_cuda_kernels_quant.cuh:131-135)
+ * output int8[n], scale float[1].  scale = max|x|/127 (1.0 for all-zero input). */
+CAIFX_API int caifx_quantize_int8_per_tensor(const float *input, void *output, void *scale, int64_t n,
+                                   caifx_stream_t stream);
+/* launch_dequantize_int8_per_tensor  (caif_cuda_kernels_quant.cuh:143-147) */
+CAIFX_API int caifx_dequantize_int8_per_tensor(const void *input, float *output, const void *scale, int64_t n,
+                                     caifx_stream_t stream);
+/* launch_quantize_int8_per_channel  (caif_cuda_kernels_quant.cuh:161-166)
+ * input [rows,cols] row-major, output int8[rows*cols], scales float[cols]. */
+CAIFX_API int caifx_quantize_int8_per_channel(const float *input, void *output, void *scales, int rows, int cols,
+                                    caifx_stream_t stream);
+/* launch_dequantize_int8_per_channel  (caif_cuda_kernels_quant.cuh:174-179) */
+CAIFX_API int caifx_dequantize_int8_per_channel(const void *input, float *output, const void *scales, int rows,
+                                      int cols, caifx_stream_t stream);
+/* launch_quantize_to_int4  (caif_cuda_kernels_quant.cuh:219-224)
+ * packed_output uint8[(n+1)/2], scales_output fp16[ceil(n/group_size)].
+ * group_size must be even when there is more than one group: with an odd size
+ * neighbouring groups share a byte and the reference's result is a data race. */
+CAIFX_API int caifx_quantize_to_int4(const float *input, void *packed_output, void *scales_output,
+                           int64_t num_elements, int group_size, caifx_stream_t stream);
+/* launch_dequantize_int4  (caif_cuda_kernels_quant.cuh:199-204) */
+CAIFX_API int caifx_dequantize_int4(const void *packed_data, const void *scales, float *output,
+                          int64_t num_elements, int group_size, caifx_stream_t stream);
+
+/* ------------------------------------------------------------------------- */
+/* Seam 2: the dequantise + GEMM pairs inside the frozen layers, fused        */
+/* ------------------------------------------------------------------------- */
+
+/* Forward of CAIF_DeviceFrozenLinear::ForwardImpl
+ * (src/caif_device_frozen_linear.cpp:412-509): replaces ConvertToComputeDtype()
+ * + input.To(ComputeT) + cublasGemmEx / CAIF_Ops::MatMulTransposeB.
+ *   Y[M,N] = cast<compute>(X)[M,K] * cast<compute>(dequant(W))[N,K]^T, fp32 accumulate.
+ * x: [M,K] of x_dtype.  y: [M,N] of y_dtype; CAIFX_F32 is the layer's own
+ * output type (:442), F16/BF16 fold the caller's following `.To(StorageT)` cast
+ * (src/caif_device_moe_frozen_expert.cpp:119-126) into the store and give the
+ * same bits as writing fp32 and casting.
+ * compute_dtype is the layer's ComputeT.  No dense copy of W is ever written. */
+CAIFX_API int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K,
+                          const void *x, int x_dtype, int compute_dtype,
+                          const void *wq, int w_kind, const void *scales, int64_t scale_period,
+                          int group_size,
+                          void *y, int y_dtype,
+                          void *workspace, size_t workspace_bytes, caifx_stream_t stream);
+
+/* Input gradient of CAIF_DeviceFrozenLinear::BackwardImpl
+ * (src/caif_device_frozen_linear.cpp:549-645): replaces ConvertToComputeDtype()
+ * + grad.To(ComputeT) + cublasGemmEx / CAIF_Ops::MatMul.
+ *   dX[M,K] = cast<compute>(dY)[M,N] * cast<compute>(dequant(W))[N,K], fp32 accumulate. */
+CAIFX_API int caifx_qlinear_backward_input(int64_t M, int64_t N, int64_t K,
+                                 const void *dy, int dy_dtype, int compute_dtype,
+                                 const void *wq, int w_kind, const void *scales, int64_t scale_period,
+                                 int group_size,
+                                 void *dx, int dx_dtype,
+                                 void *workspace, size_t workspace_bytes, caifx_stream_t stream);
+
+/* Bytes of workspace the two calls above need for this problem (may be 0).
+ * backward != 0 asks for caifx_qlinear_backward_input. */
+CAIFX_API size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtype, int compute_dtype,
+                                     int w_kind, int backward);
+
+/* The per-expert loop of CAIF_DeviceMoELayer over frozen experts
+ * (src/caif_device_moe_layer.cpp:534-557 forward, :754-778 backward) as ONE
+ * launch: expert e owns rows [offsets[e], offsets[e+1]) of the token-sorted
+ * buffer that MoEDispatchGPU packs (src/caif_cuda_kernels_moe.cu:616-647,
+ * offsets from src/caif_ops_device.cpp:4910-4919) and its own frozen weight.
+ *   forward : y[r,:] = x[r,:] * W_e^T      x [total_rows,K], y [total_rows,N]
+ *   backward: dx[r,:] = dy[r,:] * W_e      dy [total_rows,N], dx [total_rows,K]
+ * offsets: device int32[E+1], non-decreasing, offsets[E] <= total_rows (rows
+ * past offsets[E] are left untouched).  wq_ptrs / scales_ptrs: device arrays of
+ * E device pointers (one frozen linear per expert, each its own allocation as
+ * in the reference); every expert shares N, K, kind, scale_period, group_size. */
+CAIFX_API int caifx_qlinear_grouped_forward(int num_experts, const int32_t *offsets, int64_t total_rows,
+                                  int64_t N, int64_t K,
+                                  const void *x, int x_dtype, int compute_dtype,
+                                  const void *const *wq_ptrs, int w_kind,
+                                  const void *const *scales_ptrs, int64_t scale_period, int group_size,
+                                  void *y, int y_dtype,
+                                  void *workspace, size_t workspace_bytes, caifx_stream_t stream);
+CAIFX_API int caifx_qlinear_grouped_backward_input(int num_experts, const int32_t *offsets, int64_t total_rows,
+                                         int64_t N, int64_t K,
+                                         const void *dy, int dy_dtype, int compute_dtype,
+                                         const void *const *wq_ptrs, int w_kind,
+                                         const void *const *scales_ptrs, int64_t scale_period,
+                                         int group_size,
+                                         void *dx, int dx_dtype,
+                                         void *workspace, size_t workspace_bytes, caifx_stream_t stream);
+CAIFX_API size_t caifx_qlinear_grouped_workspace_bytes(int num_experts, int64_t total_rows, int64_t N, int64_t K,
+                                             int x_dtype, int compute_dtype, int w_kind, int backward);
+
+/* ------------------------------------------------------------------------- */
+/* Element-wise ops between the expert GEMMs (CAIF_DeviceMoEFrozenExpert)     */
+/* ------------------------------------------------------------------------- */
+
+/* CAIF_Ops::SiLU -> swish_forward_kernel (src/caif_cuda_kernels_activations.cu:499-532):
+ * out = T(x / (1 + expf(-x))), fp32 math, one rounding to `dtype`. */
+CAIFX_API int caifx_silu(const void *input, void *output, int64_t n, int dtype, caifx_stream_t stream);
+/* CAIF_Ops::SiLUBackward -> swish_backward_kernel (src/caif_cuda_kernels_activations.cu:539-582):
+ * s = 1/(1+expf(-x)); grad_input = T(g * s * (1 + x * (1 - s))). */
+CAIFX_API int caifx_silu_backward(const void *input, const void *grad_output, void *grad_input, int64_t n,
+                        int dtype, caifx_stream_t stream);
+/* CAIF_Ops::Multiply (src/caif_cuda_kernels_elementwise.cu:247-269): out = T(float(a) * float(b)). */
+CAIFX_API int caifx_multiply(const void *a, const void *b, void *output, int64_t n, int dtype,
+                   caifx_stream_t stream);
+/* CAIF_Ops::Add (src/caif_cuda_kernels_elementwise.cu:42-64): out = T(float(a) + float(b)). */
+CAIFX_API int caifx_add(const void *a, const void *b, void *output, int64_t n, int dtype, caifx_stream_t stream);
+/* SiLU followed by Multiply as CAIF_DeviceMoEFrozenExpert::ForwardImpl chains them
+ * (src/caif_device_moe_frozen_expert.cpp:148-153): hidden = T(float(T(silu(gate))) * float(up)).
+ * The intermediate rounding of silu(gate) to T is kept, so the bits equal the two-op sequence. */
+CAIFX_API int caifx_silu_multiply(const void *gate, const void *up, void *hidden, int64_t n, int dtype,
+                        caifx_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CAIFX_H */

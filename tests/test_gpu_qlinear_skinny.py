@@ -1,0 +1,92 @@
+"""GPU parity of the decode-regime dequant-GEMM (M <= 16) against the CPU oracle.
+
+Tolerance (north star): max relative error <= 1e-2 for bf16/fp16 compute with fp32
+accumulation, <= 1e-4 for the fp32 path; both relative to max|ref| as the reference's own
+parity tests normalise.  Measured errors are ~1e-6 because the weights fed to the matrix
+cores are bit-identical to the oracle's and only the summation order differs, so the
+asserts below use much tighter bounds than the contract.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from caif_amd import torch_ops as T                                  # noqa: E402
+from gpu_helpers import dev_as, host, make_weight, max_rel_err        # noqa: E402
+
+TOL_16 = 1e-2      # contract
+TOL_32 = 1e-4      # contract
+TIGHT_16 = 2e-5    # what identical operands + fp32 accumulation actually give
+
+
+def _check(orc, rng, M, N, K, kind, cd, xd, group=128, yd=0):
+    ow, dw = make_weight(orc, rng, N, K, kind, group)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    xt = dev_as(x, xd)
+    y = host(T.qlinear_forward(xt, dw, cd, yd))
+    want = orc.frozen_linear_forward(host(xt), ow, cd)
+    if yd != 0:
+        want = orc.round_to_dtype(want, yd)
+    err = max_rel_err(y, want)
+    bound = TOL_32 if cd == 0 else TOL_16
+    assert err <= bound, (M, N, K, kind, cd, xd, err)
+    if cd != 0 and yd == 0:
+        assert err <= TIGHT_16, (M, N, K, kind, cd, xd, err)
+    return err
+
+
+@pytest.mark.parametrize("kind", ["int4", "int8pc", "int8pt", "int8raw"])
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_decode_shapes_bf16(orc, kind, M):
+    # BASELINE config 2 geometry at reduced N (the oracle GEMM is O(M N K) on the CPU)
+    _check(orc, np.random.default_rng(M), M, 1792, 4096, kind, cd=2, xd=2)
+
+
+@pytest.mark.parametrize("kind", ["int4", "int8pc"])
+def test_decode_full_width_m1(orc, kind):
+    _check(orc, np.random.default_rng(17), 1, 14336, 4096, kind, cd=2, xd=2)
+
+
+@pytest.mark.parametrize("cd,xd", [(2, 0), (2, 1), (1, 1), (1, 2), (1, 0)])
+@pytest.mark.parametrize("kind", ["int4", "int8pc"])
+def test_dtype_mixes(orc, kind, cd, xd):
+    _check(orc, np.random.default_rng(cd * 3 + xd), 3, 256, 1024, kind, cd, xd)
+
+
+@pytest.mark.parametrize("N,K,M", [(16, 128, 1), (24, 256, 2), (1000, 384, 5), (4096, 4096, 16), (48, 8192, 7),
+                                   (1408, 2048, 13), (2048, 1408, 16)])
+def test_ragged_and_wave_count_variants(orc, N, K, M):
+    rng = np.random.default_rng(N + K + M)
+    _check(orc, rng, M, N, K, "int4", 2, 2)
+    _check(orc, rng, M, N, K, "int8pc", 2, 2)
+
+
+@pytest.mark.parametrize("group", [32, 64, 256])
+def test_int4_group_sizes(orc, group):
+    _check(orc, np.random.default_rng(group), 2, 128, 1024, "int4", 2, 2, group=group)
+
+
+@pytest.mark.parametrize("yd", [1, 2])
+def test_fused_output_cast_equals_cast_of_fp32(orc, yd):
+    _check(orc, np.random.default_rng(yd), 4, 512, 1024, "int8pc", 2, 2, yd=yd)
+
+
+def test_m1_equals_row0_of_m16(orc):
+    rng = np.random.default_rng(5)
+    ow, dw = make_weight(orc, rng, 512, 2048, "int4")
+    x = dev_as(rng.normal(0, 1, (16, 2048)), 2)
+    y16 = host(T.qlinear_forward(x, dw, 2))
+    y1 = host(T.qlinear_forward(x[:1].contiguous(), dw, 2))
+    assert np.array_equal(y16[0], y1[0])
+
+
+def test_one_hot_reads_a_weight_column_exactly(orc):
+    # X = e_j  =>  Y[0, n] = W[n, j] in the compute dtype, exactly (a single non-zero product)
+    rng = np.random.default_rng(6)
+    for kind in ("int4", "int8pc"):
+        ow, dw = make_weight(orc, rng, 320, 1024, kind)
+        for j in (0, 1, 127, 128, 777, 1023):
+            e = np.zeros((1, 1024), np.float32)
+            e[0, j] = 1.0
+            y = host(T.qlinear_forward(dev_as(e, 2), dw, 2))
+            assert np.array_equal(y[0], ow.compute_weight(2)[:, j]), (kind, j)
