@@ -1,0 +1,841 @@
+// Decode-regime dequant-GEMV for M <= 4 activation rows, streaming every weight row linearly.
+//
+// Why a second decode kernel: on MI355X a plain linear read of the 29 MB int4 weight of the
+// K=4096 x N=14336 case takes about 6 us, and any pattern that touches 64-byte pieces of 16
+// different rows per instruction is 20-50 % slower than that.  Here one load instruction of a
+// wave covers 1 KiB of ONE weight row (lane l reads bytes [16 l, 16 l + 16)), a wave walks a
+// few whole rows, and a lane keeps 8 such loads in flight.
+//
+// The matrix core still does the multiply-adds.  v_mfma_f32_16x16x32 wants, per lane
+// (i = lane%16, c = lane/16), 8 consecutive-k values of "row i" of A and of "column i" of B.
+// Here A's 16 rows are 16 different k-segments of the same weight row and B's 16 columns are the
+// same 16 k-segments of the activation row: lane l holds the codes of k-slot l in A and the
+// activations of k-slot l in B, and D[i][i] = sum over the 4 lanes (c) of segment i.  Only the
+// diagonal of D is meaningful; the other 240 products are wasted matrix-core work, which is
+// free here (the kernel is bound by HBM and by the VALU work of unpacking, not by MFMA rate).
+// Each extra activation row costs one more MFMA per step with its own B.
+//
+//   int4 (group_size % 128 == 0): a k-slot is 32 codes, segment i of a 2048-k chunk is exactly
+//     one 128-k scale group, so D[i][i] is a per-group sum of (code+136 or code+1032) * x and
+//     the lane holding it applies  scale * (D[i][i] - offset * sum_k x)  -- the post-scaled form
+//     (see caifx_gemv.hip for the numerics note).
+//   int8: a k-slot is 16 codes; float(code)*scale is rounded to the compute dtype exactly as
+//     the reference does.  With per-channel scales the index (n*K+k) % period depends on the
+//     row only through (n*K) % period, so a wave takes rows of one residue class
+//     n = v + V*i (V = period / gcd(K, period)) and keeps that class's scales in registers.
+#include "caifx_internal.hpp"
+
+namespace caifx {
+namespace {
+
+template <typename CT> struct Mfma16;
+template <> struct Mfma16<bf16_t> {
+  typedef bf16x8_t vec_t;
+  static constexpr uint32_t kMagic = 0x43084308u;
+  static constexpr float kOffset = 136.0f;
+  static __device__ __forceinline__ floatx4_t run(vec_t a, vec_t b, floatx4_t c)
+  {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma16<f16_t> {
+  typedef f16x8_t vec_t;
+  static constexpr uint32_t kMagic = 0x64086408u;
+  static constexpr float kOffset = 1032.0f;
+  static __device__ __forceinline__ floatx4_t run(vec_t a, vec_t b, floatx4_t c)
+  {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+struct RowArgs {
+  const uint8_t *wq;
+  const void *scales;
+  const void *x;
+  void *y;
+  int M;
+  int y_dtype;
+  int64_t N, K;
+  int group_shift;      // int4
+  int period;           // int8 vec
+  int row_stride;       // int8 vec: V
+  int rows_per_wave;
+  int waves_per_class;  // int8: waves that share one residue class
+  int total_waves;
+  int cpr;              // chunks (one load instruction of a wave) per weight row
+  int xpitch;           // staged activations: elements per row (cpr * k-per-chunk)
+};
+
+template <typename CT, typename XT>
+__device__ __forceinline__ typename Mfma16<CT>::vec_t load_x8g(const XT *p)
+{
+  typename Mfma16<CT>::vec_t v;
+  if constexpr (sizeof(XT) == 2 && dtype_code<XT>::value == dtype_code<CT>::value) {
+    v = *reinterpret_cast<const typename Mfma16<CT>::vec_t *>(p);
+  } else if constexpr (sizeof(XT) == 4) {
+    const floatx4_t a = *reinterpret_cast<const floatx4_t *>(p);
+    const floatx4_t b = *reinterpret_cast<const floatx4_t *>(p + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[j] = from_f32<CT>(a[j]);
+      v[4 + j] = from_f32<CT>(b[j]);
+    }
+  } else {
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(p);
+    const XT *e = reinterpret_cast<const XT *>(&raw);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = from_f32<CT>(to_f32<XT>(e[j]));
+  }
+  return v;
+}
+
+// v + (v moved across lanes by DPP control kCtrl); lanes outside kRowMask add 0
+template <int kCtrl, int kRowMask = 0xF>
+__device__ __forceinline__ float dpp_add(float v)
+{
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, kRowMask, 0xF, false);
+  return v + __builtin_bit_cast(float, moved);
+}
+
+// sum over each aligned group of 16 lanes, result in all 16 (4 VALU ops, no LDS)
+__device__ __forceinline__ float row16_sum(float v)
+{
+  v = dpp_add<0xB1>(v);    // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E>(v);    // quad_perm [2,3,0,1]
+  v = dpp_add<0x141>(v);   // row_half_mirror
+  v = dpp_add<0x140>(v);   // row_mirror
+  return v;
+}
+
+// sum over the wave; valid in lanes 48..63 (read it from lane 63)
+__device__ __forceinline__ float wave_sum_hi(float v)
+{
+  v = row16_sum(v);
+  v = dpp_add<0x142, 0xA>(v);   // row_bcast:15 into rows 1 and 3
+  v = dpp_add<0x143, 0xC>(v);   // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+__device__ __forceinline__ void store_y(void *y, int y_dtype, int64_t o, float v)
+{
+  if (y_dtype == CAIFX_F32) static_cast<float *>(y)[o] = v;
+  else if (y_dtype == CAIFX_BF16) static_cast<bf16_t *>(y)[o] = from_f32<bf16_t>(v);
+  else static_cast<f16_t *>(y)[o] = from_f32<f16_t>(v);
+}
+
+// D[i][i] of the 16x16 tile lives on lane i + 16*(i/4) in element i%4; other lanes return 0.
+__device__ __forceinline__ float diag_of(floatx4_t d, int lane)
+{
+  const int r = lane & 15;
+  const int t = r & 3;
+  float v = d[0];
+  v = (t == 1) ? d[1] : v;
+  v = (t == 2) ? d[2] : v;
+  v = (t == 3) ? d[3] : v;
+  return ((lane >> 4) == (r >> 2)) ? v : 0.0f;
+}
+
+// Stage X[MT rows][K] as compute-dtype values into LDS, zero padded to `xpitch` per row, in the
+// order the MFMA B operand is read: row m is a sequence of 1 KiB blocks (chunk, step j), and in
+// each block lane l owns 16 bytes at l*16, so the ds_read_b128 of a wave is conflict free.
+// kInt4: a k-slot is 32 values (4 steps), the slot of lane l is 4*(l%16) + l/16, every aligned
+// run of 8 is stored in the order 0,4,1,5,2,6,3,7 and the per-128-k sums of the rounded values
+// go to xsum[m][xpitch/128].  Otherwise (int8): a k-slot is 16 values (2 steps), slot = lane.
+template <typename CT, typename XT, int MT, bool kInt4>
+__device__ __forceinline__ void stage_x(const RowArgs &a, CT *xs, float *xsum)
+{
+  typedef typename Mfma16<CT>::vec_t vec_t;
+  constexpr int kSteps = kInt4 ? 4 : 2;
+  const XT *xg = static_cast<const XT *>(a.x);
+  const int lane = threadIdx.x & 63;
+  const int per_row = a.xpitch / 8;                      // 8-element pieces per staged row
+  for (int p = threadIdx.x; p < MT * per_row; p += blockDim.x) {
+    const int m = p / per_row;
+    const int piece = p - m * per_row;
+    const int k = piece * 8;
+    const int msrc = m < a.M ? m : a.M - 1;
+    vec_t v;
+    if (k < a.K) {
+      v = load_x8g<CT, XT>(xg + static_cast<int64_t>(msrc) * a.K + k);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = from_f32<CT>(0.0f);
+    }
+    const int j = piece % kSteps;
+    const int slot_all = piece / kSteps;                 // chunk*64 + slot
+    const int chunk = slot_all >> 6;
+    const int slot = slot_all & 63;
+    int l = slot;
+    if constexpr (kInt4) {
+      l = (slot & 3) * 16 + (slot >> 2);
+      float part = 0.0f;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) part += to_f32<CT>(v[t]);
+      part = row16_sum(part);
+      if ((lane & 15) == 0) xsum[m * (a.xpitch >> 7) + (k >> 7)] = part;
+      vec_t q;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        q[2 * t] = v[t];
+        q[2 * t + 1] = v[t + 4];
+      }
+      v = q;
+    }
+    *reinterpret_cast<vec_t *>(xs + m * a.xpitch + ((chunk * kSteps + j) * 64 + l) * 8) = v;
+  }
+}
+
+// ------------------------------------------------------------------ int4, post-scaled
+template <typename CT, typename XT, int MT>
+__global__ __launch_bounds__(256) void rowlin_int4_kernel(RowArgs a)
+{
+  typedef typename Mfma16<CT>::vec_t vec_t;
+  constexpr int U = 8;                                   // 16-byte loads in flight per lane
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int groups_pad = a.xpitch >> 7;
+  float *xsum = reinterpret_cast<float *>(smem);                        // [MT][groups_pad]
+  CT *xs = reinterpret_cast<CT *>(xsum + ((MT * groups_pad + 3) & ~3)); // [MT][xpitch]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int gw = blockIdx.x * 4 + wave;
+  const int64_t row0 = static_cast<int64_t>(gw) * a.rows_per_wave;
+  int nrows = 0;
+  if (row0 < a.N) nrows = static_cast<int>(a.N - row0 < a.rows_per_wave ? a.N - row0 : a.rows_per_wave);
+  const int cpr = a.cpr;
+  const int ntasks = nrows * cpr;
+  const int slots = static_cast<int>(a.K >> 5);          // 32-code slots per row
+  const int64_t rowbytes = a.K >> 1;
+  const bool is_diag = (lane >> 4) == ((lane & 15) >> 2);
+  const int di = lane & 15;
+  const int pslot = (lane & 15) * 4 + (lane >> 4);       // k-slot of this lane inside a chunk
+
+  u32x4_t wreg[U];
+  f16_t sreg[U];
+  // task t = (row t / cpr, chunk t % cpr); keep the issue cursor incrementally
+  int irow = 0, ichunk = 0;
+  auto issue = [&](int u) {
+    const int slot = ichunk * 64 + pslot;
+    u32x4_t w = {0u, 0u, 0u, 0u};
+    if (slot < slots)
+      w = *reinterpret_cast<const u32x4_t *>(a.wq + (row0 + irow) * rowbytes + static_cast<int64_t>(slot) * 16);
+    wreg[u] = w;
+    f16_t s = static_cast<f16_t>(0.0f);
+    const int gslot = ichunk * 64 + di * 4;              // first slot of the group this lane's diagonal covers
+    if (is_diag && gslot < slots)
+      s = static_cast<const f16_t *>(a.scales)[((row0 + irow) * a.K + (static_cast<int64_t>(gslot) << 5)) >> a.group_shift];
+    sreg[u] = s;
+    if (++ichunk == cpr) {
+      ichunk = 0;
+      ++irow;
+    }
+  };
+
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    if (u < ntasks) issue(u);
+
+  stage_x<CT, XT, MT, true>(a, xs, xsum);
+  __syncthreads();
+
+  float tot[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) tot[m] = 0.0f;
+  int crow = 0, cchunk = 0;
+  for (int t0 = 0; t0 < ntasks; t0 += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int t = t0 + u;
+      if (t < ntasks) {
+        const u32x4_t w = wreg[u];
+        const float s = to_f32(sreg[u]);
+        if (t + U < ntasks) issue(u);
+        floatx4_t part[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) part[m] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        const CT *xb = xs + (cchunk * 4 * 64 + lane) * 8;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          u32x4_t c4;
+          const uint32_t p = w[j];
+          c4[0] = (p & 0x000F000Fu) ^ Mfma16<CT>::kMagic;           // codes 0,4
+          c4[1] = ((p >> 4) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;    // codes 1,5
+          c4[2] = ((p >> 8) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;    // codes 2,6
+          c4[3] = ((p >> 12) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;   // codes 3,7
+          const vec_t av = *reinterpret_cast<const vec_t *>(&c4);
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            const vec_t bv = *reinterpret_cast<const vec_t *>(xb + m * a.xpitch + j * 64 * 8);
+            part[m] = Mfma16<CT>::run(av, bv, part[m]);
+          }
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const float corr = Mfma16<CT>::kOffset * xsum[m * groups_pad + cchunk * 16 + di];
+          tot[m] = __builtin_fmaf(s, diag_of(part[m], lane) - corr, tot[m]);
+        }
+        if (++cchunk == cpr) {
+          cchunk = 0;
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            const float v = wave_sum_hi(tot[m]);
+            if (lane == 63 && m < a.M) store_y(a.y, a.y_dtype, static_cast<int64_t>(m) * a.N + row0 + crow, v);
+            tot[m] = 0.0f;
+          }
+          ++crow;
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------ fixed-shape fast paths
+// Same arithmetic as the kernels above for rows made of whole chunks (K = CPR * 2048 for int4,
+// CPR * 1024 for int8).  Every inner trip count is a compile-time constant; the activations are
+// requested BEFORE the first weight loads so that staging them does not wait for the weights
+// (loads return in order); a wave walks `rows_per_wave` rows through a ring of 8/CPR rows in
+// flight, so unpacking one row overlaps the HBM latency of the next ones.
+
+// Activation pieces (8 values) a thread stages: piece p = threadIdx.x + i*256 of MT*PIECES_PER_ROW.
+template <typename CT, int MT, int kPiecesPerRow>
+struct XPieces {
+  static constexpr int kTotal = MT * kPiecesPerRow;
+  static constexpr int kPerThread = (kTotal + 255) / 256;
+  typename Mfma16<CT>::vec_t v[kPerThread];
+};
+
+template <typename CT, int MT, int kPiecesPerRow>
+__device__ __forceinline__ void x_request(const RowArgs &a, XPieces<CT, MT, kPiecesPerRow> &xp)
+{
+  typedef typename Mfma16<CT>::vec_t vec_t;
+  const CT *xg = static_cast<const CT *>(a.x);
+#pragma unroll
+  for (int i = 0; i < XPieces<CT, MT, kPiecesPerRow>::kPerThread; ++i) {
+    const int p = threadIdx.x + i * 256;
+    const int m = p / kPiecesPerRow;
+    const int piece = p - m * kPiecesPerRow;
+    const int msrc = m < a.M ? m : a.M - 1;
+    if (p < MT * kPiecesPerRow)
+      xp.v[i] = *reinterpret_cast<const vec_t *>(xg + static_cast<int64_t>(msrc) * a.K + piece * 8);
+  }
+}
+
+template <typename CT, int MT, int kPiecesPerRow, bool kInt4>
+__device__ __forceinline__ void x_commit(const XPieces<CT, MT, kPiecesPerRow> &xp, CT *xs, float *xsum)
+{
+  typedef typename Mfma16<CT>::vec_t vec_t;
+  constexpr int kSteps = kInt4 ? 4 : 2;
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int i = 0; i < XPieces<CT, MT, kPiecesPerRow>::kPerThread; ++i) {
+    const int p = threadIdx.x + i * 256;
+    if (p < MT * kPiecesPerRow) {
+      const int m = p / kPiecesPerRow;
+      const int piece = p - m * kPiecesPerRow;
+      vec_t v = xp.v[i];
+      const int j = piece % kSteps;
+      const int slot_all = piece / kSteps;
+      const int chunk = slot_all >> 6;
+      const int slot = slot_all & 63;
+      int l = slot;
+      if constexpr (kInt4) {
+        l = (slot & 3) * 16 + (slot >> 2);
+        float part = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) part += to_f32<CT>(v[t]);
+        part = row16_sum(part);
+        if ((lane & 15) == 0) xsum[m * (kPiecesPerRow / 16) + (piece >> 4)] = part;
+        vec_t q;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          q[2 * t] = v[t];
+          q[2 * t + 1] = v[t + 4];
+        }
+        v = q;
+      }
+      *reinterpret_cast<vec_t *>(xs + m * (kPiecesPerRow * 8) + ((chunk * kSteps + j) * 64 + l) * 8) = v;
+    }
+  }
+}
+
+template <typename CT, int MT, int CPR>
+__global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
+{
+  typedef typename Mfma16<CT>::vec_t vec_t;
+  constexpr int D = 8 / CPR;                 // rows in flight
+  constexpr int kPieces = CPR * 256;         // 8-value pieces per activation row
+  constexpr int kGroupsPad = CPR * 16;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float *xsum = reinterpret_cast<float *>(smem);                        // [MT][CPR*16]
+  CT *xs = reinterpret_cast<CT *>(xsum + ((MT * kGroupsPad + 3) & ~3)); // [MT][CPR*2048]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * a.rows_per_wave;
+  int nrows = 0;
+  if (row0 < a.N) nrows = static_cast<int>(a.N - row0 < a.rows_per_wave ? a.N - row0 : a.rows_per_wave);
+  const bool is_diag = (lane >> 4) == ((lane & 15) >> 2);
+  const int di = lane & 15;
+  const int pslot = di * 4 + (lane >> 4);
+  constexpr int64_t kRowBytes = static_cast<int64_t>(CPR) * 1024;
+  const int groups_per_row = (CPR * 2048) >> a.group_shift;
+
+  XPieces<CT, MT, kPieces> xp;
+  x_request<CT, MT, kPieces>(a, xp);
+
+  const uint8_t *wp = a.wq + row0 * kRowBytes + pslot * 16;
+  const f16_t *sp = static_cast<const f16_t *>(a.scales) + row0 * groups_per_row;
+  u32x4_t w[D][CPR];
+  f16_t sc[D][CPR];
+  auto issue = [&](int d, int r) {
+#pragma unroll
+    for (int c = 0; c < CPR; ++c) {
+      w[d][c] = *reinterpret_cast<const u32x4_t *>(wp + r * kRowBytes + c * 1024);
+      sc[d][c] = sp[r * groups_per_row + ((c * 2048 + di * 128) >> a.group_shift)];
+    }
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < nrows) issue(d, d);
+
+  x_commit<CT, MT, kPieces, true>(xp, xs, xsum);
+  __syncthreads();
+
+  float corr[MT][CPR];
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int c = 0; c < CPR; ++c) corr[m][c] = Mfma16<CT>::kOffset * xsum[m * kGroupsPad + c * 16 + di];
+  const int tsel = di & 3;
+
+  for (int r0 = 0; r0 < nrows; r0 += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int r = r0 + d;
+      if (r < nrows) {
+        u32x4_t wr[CPR];
+        float sr[CPR];
+#pragma unroll
+        for (int c = 0; c < CPR; ++c) {
+          wr[c] = w[d][c];
+          sr[c] = to_f32(sc[d][c]);
+        }
+        if (r + D < nrows) issue(d, r + D);
+        float tot[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) tot[m] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CPR; ++c) {
+          floatx4_t part[MT];
+#pragma unroll
+          for (int m = 0; m < MT; ++m) part[m] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            u32x4_t c4;
+            const uint32_t p = wr[c][j];
+            c4[0] = (p & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
+            c4[1] = ((p >> 4) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
+            c4[2] = ((p >> 8) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
+            c4[3] = ((p >> 12) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
+            const vec_t av = *reinterpret_cast<const vec_t *>(&c4);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+              const vec_t bv = *reinterpret_cast<const vec_t *>(xs + m * (CPR * 2048) + ((c * 4 + j) * 64 + lane) * 8);
+              part[m] = Mfma16<CT>::run(av, bv, part[m]);
+            }
+          }
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            float dsel = part[m][0];
+            dsel = (tsel == 1) ? part[m][1] : dsel;
+            dsel = (tsel == 2) ? part[m][2] : dsel;
+            dsel = (tsel == 3) ? part[m][3] : dsel;
+            tot[m] = __builtin_fmaf(sr[c], dsel - corr[m][c], tot[m]);
+          }
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const float v = wave_sum_hi(is_diag ? tot[m] : 0.0f);
+          if (lane == 63 && m < a.M) store_y(a.y, a.y_dtype, static_cast<int64_t>(m) * a.N + row0 + r, v);
+        }
+      }
+    }
+  }
+}
+
+template <typename CT, int MT, bool kVec, int CPR>
+__global__ __launch_bounds__(256) void rowlin_int8_fast_kernel(RowArgs a)
+{
+  typedef typename Mfma16<CT>::vec_t vec_t;
+  constexpr int D = 8 / CPR;                 // rows in flight
+  constexpr int kPieces = CPR * 128;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  CT *xs = reinterpret_cast<CT *>(smem);     // [MT][CPR*1024]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int gw = blockIdx.x * 4 + wave;
+  const int cls = gw / a.waves_per_class;
+  const int64_t i0 = static_cast<int64_t>(gw - cls * a.waves_per_class) * a.rows_per_wave;
+  const int64_t V = a.row_stride;
+  int nrows = 0;
+  if (gw < a.total_waves) {
+    const int64_t first = cls + V * i0;
+    if (first < a.N) {
+      const int64_t avail = (a.N - first + V - 1) / V;
+      nrows = static_cast<int>(avail < a.rows_per_wave ? avail : a.rows_per_wave);
+    }
+  }
+  constexpr int64_t kRowBytes = static_cast<int64_t>(CPR) * 1024;
+
+  XPieces<CT, MT, kPieces> xp;
+  x_request<CT, MT, kPieces>(a, xp);
+
+  const uint8_t *wp = a.wq + (cls + V * i0) * kRowBytes + lane * 16;
+  const int64_t rstep = V * kRowBytes;
+  u32x4_t w[D][CPR];
+  auto issue = [&](int d, int r) {
+#pragma unroll
+    for (int c = 0; c < CPR; ++c) w[d][c] = *reinterpret_cast<const u32x4_t *>(wp + r * rstep + c * 1024);
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < nrows) issue(d, d);
+
+  floatx4_t sc[CPR][4];
+  float s_scalar = 1.0f;
+  if constexpr (kVec) {
+    const float *sp = static_cast<const float *>(a.scales);
+#pragma unroll
+    for (int c = 0; c < CPR; ++c) {
+      const int idx = static_cast<int>((static_cast<int64_t>(cls) * (CPR * 1024) + (c * 64 + lane) * 16) % a.period);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        int i = idx + 4 * q;
+        if (i >= a.period) i -= a.period;
+        sc[c][q] = *reinterpret_cast<const floatx4_t *>(sp + i);
+      }
+    }
+  } else {
+    if (a.scales) s_scalar = static_cast<const float *>(a.scales)[0];
+  }
+
+  x_commit<CT, MT, kPieces, false>(xp, xs, nullptr);
+  __syncthreads();
+
+  for (int r0 = 0; r0 < nrows; r0 += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int r = r0 + d;
+      if (r < nrows) {
+        u32x4_t wr[CPR];
+#pragma unroll
+        for (int c = 0; c < CPR; ++c) wr[c] = w[d][c];
+        if (r + D < nrows) issue(d, r + D);
+        floatx4_t acc[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[m] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < CPR; ++c) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            float lo[4], hi[4];
+            int8x4_to_f32(wr[c][2 * j], lo);
+            int8x4_to_f32(wr[c][2 * j + 1], hi);
+            vec_t av;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float s0 = kVec ? sc[c][2 * j][q] : s_scalar;
+              const float s1 = kVec ? sc[c][2 * j + 1][q] : s_scalar;
+              av[q] = from_f32<CT>(lo[q] * s0);
+              av[4 + q] = from_f32<CT>(hi[q] * s1);
+            }
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+              const vec_t bv = *reinterpret_cast<const vec_t *>(xs + m * (CPR * 1024) + ((c * 2 + j) * 64 + lane) * 8);
+              acc[m] = Mfma16<CT>::run(av, bv, acc[m]);
+            }
+          }
+        }
+        const int64_t nrow = cls + V * (i0 + r);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const float v = wave_sum_hi(diag_of(acc[m], lane));
+          if (lane == 63 && m < a.M) store_y(a.y, a.y_dtype, static_cast<int64_t>(m) * a.N + nrow, v);
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------ int8, exact
+// kVec: per-channel scales (period > 1) cached in registers per residue class.
+template <typename CT, typename XT, int MT, bool kVec, int CPR>
+__global__ __launch_bounds__(256) void rowlin_int8_kernel(RowArgs a)
+{
+  typedef typename Mfma16<CT>::vec_t vec_t;
+  constexpr int RB = (CPR == 1) ? 8 : (CPR == 2 ? 4 : 2);   // rows in flight (RB*CPR 16-byte loads per lane)
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  CT *xs = reinterpret_cast<CT *>(smem);                    // [MT][xpitch]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int gw = blockIdx.x * 4 + wave;
+  const int cls = gw / a.waves_per_class;                   // residue class v (0 when row_stride == 1)
+  const int64_t i0 = static_cast<int64_t>(gw - cls * a.waves_per_class) * a.rows_per_wave;
+  const int64_t V = a.row_stride;
+  // rows of this wave: n = cls + V * (i0 + t), t < nrows
+  int nrows = 0;
+  if (gw < a.total_waves) {
+    const int64_t first = cls + V * i0;
+    if (first < a.N) {
+      const int64_t avail = (a.N - first + V - 1) / V;
+      nrows = static_cast<int>(avail < a.rows_per_wave ? avail : a.rows_per_wave);
+    }
+  }
+  const int slots = static_cast<int>(a.K >> 4);             // 16-code slots per row
+
+  // scales of this residue class for this lane's slots
+  floatx4_t sc[CPR][4];
+  float s_scalar = 1.0f;
+  if constexpr (kVec) {
+    const float *sp = static_cast<const float *>(a.scales);
+#pragma unroll
+    for (int c = 0; c < CPR; ++c) {
+      const int slot = c * 64 + lane;
+      const int64_t k0 = static_cast<int64_t>(slot < slots ? slot : 0) << 4;
+      int idx = static_cast<int>((static_cast<int64_t>(cls) * a.K + k0) % a.period);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        int i = idx + 4 * q;
+        if (i >= a.period) i -= a.period;
+        sc[c][q] = *reinterpret_cast<const floatx4_t *>(sp + i);
+      }
+    }
+  } else {
+    if (a.scales) s_scalar = static_cast<const float *>(a.scales)[0];
+  }
+
+  u32x4_t wreg[RB][CPR];
+  auto issue = [&](int rb, int t) {
+    const uint8_t *rowp = a.wq + (cls + V * (i0 + t)) * a.K;
+#pragma unroll
+    for (int c = 0; c < CPR; ++c) {
+      const int slot = c * 64 + lane;
+      u32x4_t w = {0u, 0u, 0u, 0u};
+      if (slot < slots) w = *reinterpret_cast<const u32x4_t *>(rowp + static_cast<int64_t>(slot) * 16);
+      wreg[rb][c] = w;
+    }
+  };
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+    if (rb < nrows) issue(rb, rb);
+
+  stage_x<CT, XT, MT, false>(a, xs, nullptr);
+  __syncthreads();
+
+  for (int t0 = 0; t0 < nrows; t0 += RB) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const int t = t0 + rb;
+      if (t < nrows) {
+        u32x4_t w[CPR];
+#pragma unroll
+        for (int c = 0; c < CPR; ++c) w[c] = wreg[rb][c];
+        if (t + RB < nrows) issue(rb, t + RB);
+        floatx4_t acc[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[m] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < CPR; ++c) {
+          const CT *xb = xs + (c * 2 * 64 + lane) * 8;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            float lo[4], hi[4];
+            int8x4_to_f32(w[c][2 * j], lo);
+            int8x4_to_f32(w[c][2 * j + 1], hi);
+            vec_t av;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float s0 = kVec ? sc[c][2 * j][q] : s_scalar;
+              const float s1 = kVec ? sc[c][2 * j + 1][q] : s_scalar;
+              av[q] = from_f32<CT>(lo[q] * s0);
+              av[4 + q] = from_f32<CT>(hi[q] * s1);
+            }
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+              const vec_t bv = *reinterpret_cast<const vec_t *>(xb + m * a.xpitch + j * 64 * 8);
+              acc[m] = Mfma16<CT>::run(av, bv, acc[m]);
+            }
+          }
+        }
+        const int64_t nrow = cls + V * (i0 + t);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const float v = wave_sum_hi(diag_of(acc[m], lane));
+          if (lane == 63 && m < a.M) store_y(a.y, a.y_dtype, static_cast<int64_t>(m) * a.N + nrow, v);
+        }
+      }
+    }
+  }
+}
+
+template <typename CT, int MT, int CPR>
+int launch_int4_fast(const RowArgs &ra, hipStream_t s)
+{
+  const size_t lds = static_cast<size_t>((MT * CPR * 16 + 3) & ~3) * 4 + static_cast<size_t>(MT) * CPR * 2048 * 2;
+  hipLaunchKernelGGL((rowlin_int4_fast_kernel<CT, MT, CPR>), dim3(static_cast<unsigned>((ra.total_waves + 3) / 4)),
+                     dim3(256), lds, s, ra);
+  return launch_status();
+}
+
+template <typename CT, int MT, bool kVec, int CPR>
+int launch_int8_fast(const RowArgs &ra, hipStream_t s)
+{
+  const size_t lds = static_cast<size_t>(MT) * CPR * 1024 * 2;
+  hipLaunchKernelGGL((rowlin_int8_fast_kernel<CT, MT, kVec, CPR>), dim3(static_cast<unsigned>((ra.total_waves + 3) / 4)),
+                     dim3(256), lds, s, ra);
+  return launch_status();
+}
+
+template <typename CT, typename XT, int MT>
+int launch_int4(const RowArgs &ra, hipStream_t s)
+{
+  if constexpr (dtype_code<XT>::value == dtype_code<CT>::value) {
+    const bool full = (ra.K % 2048 == 0);
+    if (full && ra.cpr == 1) return launch_int4_fast<CT, MT, 1>(ra, s);
+    if (full && ra.cpr == 2) return launch_int4_fast<CT, MT, 2>(ra, s);
+    if (full && ra.cpr == 4) return launch_int4_fast<CT, MT, 4>(ra, s);
+  }
+  const size_t lds = static_cast<size_t>((MT * (ra.xpitch >> 7) + 3) & ~3) * 4 + static_cast<size_t>(MT) * ra.xpitch * 2;
+  const unsigned grid = static_cast<unsigned>((ra.total_waves + 3) / 4);
+  hipLaunchKernelGGL((rowlin_int4_kernel<CT, XT, MT>), dim3(grid), dim3(256), lds, s, ra);
+  return launch_status();
+}
+
+template <typename CT, typename XT, int MT, bool kVec>
+int launch_int8(const RowArgs &ra, hipStream_t s)
+{
+  if constexpr (dtype_code<XT>::value == dtype_code<CT>::value) {
+    const bool full = (ra.K % 1024 == 0);
+    if (full && ra.cpr == 1) return launch_int8_fast<CT, MT, kVec, 1>(ra, s);
+    if (full && ra.cpr == 2) return launch_int8_fast<CT, MT, kVec, 2>(ra, s);
+    if (full && ra.cpr == 4) return launch_int8_fast<CT, MT, kVec, 4>(ra, s);
+  }
+  const size_t lds = static_cast<size_t>(MT) * ra.xpitch * 2;
+  const unsigned grid = static_cast<unsigned>((ra.total_waves + 3) / 4);
+  switch (ra.cpr) {
+    case 1: hipLaunchKernelGGL((rowlin_int8_kernel<CT, XT, MT, kVec, 1>), dim3(grid), dim3(256), lds, s, ra); break;
+    case 2: hipLaunchKernelGGL((rowlin_int8_kernel<CT, XT, MT, kVec, 2>), dim3(grid), dim3(256), lds, s, ra); break;
+    case 3: hipLaunchKernelGGL((rowlin_int8_kernel<CT, XT, MT, kVec, 3>), dim3(grid), dim3(256), lds, s, ra); break;
+    case 4: hipLaunchKernelGGL((rowlin_int8_kernel<CT, XT, MT, kVec, 4>), dim3(grid), dim3(256), lds, s, ra); break;
+    default: return CAIFX_ERR_UNSUPPORTED;
+  }
+  return launch_status();
+}
+
+template <typename CT, typename XT, int MT>
+int pick_kind(const RowArgs &ra, int kind, hipStream_t s)
+{
+  if (kind == 0) return launch_int4<CT, XT, MT>(ra, s);
+  if (kind == 1) return launch_int8<CT, XT, MT, false>(ra, s);
+  return launch_int8<CT, XT, MT, true>(ra, s);
+}
+
+template <typename CT, typename XT>
+int pick_m(const RowArgs &ra, int kind, hipStream_t s)
+{
+  if (ra.M == 1) return pick_kind<CT, XT, 1>(ra, kind, s);
+  if (ra.M == 2) return pick_kind<CT, XT, 2>(ra, kind, s);
+  return pick_kind<CT, XT, 4>(ra, kind, s);
+}
+
+template <typename CT>
+int pick_xt(const RowArgs &ra, int x_dtype, int kind, hipStream_t s)
+{
+  switch (x_dtype) {
+    case CAIFX_F32: return pick_m<CT, float>(ra, kind, s);
+    case CAIFX_F16: return pick_m<CT, f16_t>(ra, kind, s);
+    default: return pick_m<CT, bf16_t>(ra, kind, s);
+  }
+}
+
+int64_t gcd64(int64_t a, int64_t b)
+{
+  while (b) {
+    const int64_t t = a % b;
+    a = b;
+    b = t;
+  }
+  return a;
+}
+
+int pick_rows_per_wave(int64_t rows, int min_rows)
+{
+  // aim for two waves per SIMD (2048 waves): each walks its rows through a ring of loads, so
+  // unpacking overlaps the HBM latency of the rows behind it
+  int64_t rpw = (rows + 2047) / 2048;
+  if (rpw < min_rows) rpw = min_rows;
+  if (rpw > 64) rpw = 64;
+  return static_cast<int>(rpw);
+}
+
+}  // namespace
+
+int rowlin_forward(const GemmArgs &g, hipStream_t s)
+{
+  if (g.offsets || g.M < 1 || g.M > 4 || g.compute_dtype == CAIFX_F32) return CAIFX_ERR_UNSUPPORTED;
+  if (g.N < 1 || g.N > (int64_t{1} << 30) || g.K > (int64_t{1} << 20)) return CAIFX_ERR_UNSUPPORTED;
+  if (!aligned_to(g.w.q, 16) || !aligned_to(g.x, 16)) return CAIFX_ERR_UNSUPPORTED;
+  const bool int4 = g.w.kind == CAIFX_W_INT4_GROUP;
+
+  RowArgs ra{};
+  ra.wq = static_cast<const uint8_t *>(g.w.q);
+  ra.scales = g.w.scales;
+  ra.x = g.x;
+  ra.y = g.y;
+  ra.M = static_cast<int>(g.M);
+  ra.y_dtype = g.y_dtype;
+  ra.N = g.N;
+  ra.K = g.K;
+  ra.row_stride = 1;
+  const int mt = g.M == 3 ? 4 : static_cast<int>(g.M);
+  int kind;
+  if (int4) {
+    const int gs = g.w.group_size;
+    if (!g.w.scales || gs < 128 || (gs & (gs - 1)) != 0 || g.K % 128 != 0) return CAIFX_ERR_UNSUPPORTED;
+    ra.group_shift = __builtin_ctz(static_cast<unsigned>(gs));
+    kind = 0;
+    ra.cpr = static_cast<int>((g.K + 2047) / 2048);
+    ra.xpitch = ra.cpr * 2048;
+    ra.rows_per_wave = pick_rows_per_wave(g.N, (8 + ra.cpr - 1) / ra.cpr);
+    ra.total_waves = static_cast<int>((g.N + ra.rows_per_wave - 1) / ra.rows_per_wave);
+    ra.waves_per_class = ra.total_waves;
+    if (static_cast<size_t>(mt) * ra.xpitch * 2 + 4096 > 64 * 1024) return CAIFX_ERR_UNSUPPORTED;
+  } else {
+    if (g.K % 16 != 0 || g.K > 4096) return CAIFX_ERR_UNSUPPORTED;
+    ra.cpr = static_cast<int>((g.K + 1023) / 1024);
+    ra.xpitch = ra.cpr * 1024;
+    if (!g.w.scales || g.w.scale_period == 1) {
+      kind = 1;
+    } else {
+      const int64_t P = g.w.scale_period;
+      if (P % 4 != 0 || P < 16 || P > (int64_t{1} << 30) || !aligned_to(g.w.scales, 16)) return CAIFX_ERR_UNSUPPORTED;
+      kind = 2;
+      ra.period = static_cast<int>(P);
+      const int64_t V = P / gcd64(g.K % P == 0 ? P : g.K % P, P);
+      if (V * 256 > g.N) return CAIFX_ERR_UNSUPPORTED;   // too few rows per residue class to amortise the scales
+      ra.row_stride = static_cast<int>(V);
+    }
+    const int64_t rows_class = (g.N + ra.row_stride - 1) / ra.row_stride;
+    const int rb = ra.cpr == 1 ? 8 : (ra.cpr == 2 ? 4 : 2);
+    ra.rows_per_wave = pick_rows_per_wave(g.N, kind == 2 ? 2 * rb : rb);
+    ra.waves_per_class = static_cast<int>((rows_class + ra.rows_per_wave - 1) / ra.rows_per_wave);
+    ra.total_waves = ra.waves_per_class * ra.row_stride;
+    if (static_cast<size_t>(mt) * ra.xpitch * 2 > 64 * 1024) return CAIFX_ERR_UNSUPPORTED;
+  }
+  if (g.compute_dtype == CAIFX_BF16) return pick_xt<bf16_t>(ra, g.x_dtype, kind, s);
+  return pick_xt<f16_t>(ra, g.x_dtype, kind, s);
+}
+
+}  // namespace caifx

@@ -37,6 +37,8 @@ int generic_backward(const GemmArgs &a, hipStream_t s);
 // M <= 16 decode path (memory bound).  Returns CAIFX_ERR_UNSUPPORTED when the shape is outside
 // its tiling assumptions so that the caller can fall back.
 int skinny_forward(const GemmArgs &a, hipStream_t s);
+// M <= 4 decode path that streams each weight row linearly (the fastest access pattern).
+int rowlin_forward(const GemmArgs &a, hipStream_t s);
 
 // Large-M MFMA path (compute bound), forward and input gradient, plain and grouped.
 int mfma_forward(const GemmArgs &a, hipStream_t s);

@@ -2,9 +2,12 @@
 
 Tolerance (north star): max relative error <= 1e-2 for bf16/fp16 compute with fp32
 accumulation, <= 1e-4 for the fp32 path; both relative to max|ref| as the reference's own
-parity tests normalise.  Measured errors are ~1e-6 because the weights fed to the matrix
-cores are bit-identical to the oracle's and only the summation order differs, so the
-asserts below use much tighter bounds than the contract.
+parity tests normalise.  The asserts are tighter than the contract:
+  * int8 and int4 with group sizes below 128 feed the matrix cores weights that are
+    bit-identical to the oracle's, so only the summation order differs (~1e-6);
+  * int4 with group size 128 (or a multiple) is scaled after the per-group accumulation, which
+    skips the reference's bf16 rounding of code*scale: the difference is that rounding,
+    <= 2^-9 per weight with random sign, a few 1e-4 of max|ref| after the sum over K.
 """
 import numpy as np
 import pytest
@@ -17,6 +20,7 @@ from gpu_helpers import dev_as, host, make_weight, max_rel_err        # noqa: E4
 TOL_16 = 1e-2      # contract
 TOL_32 = 1e-4      # contract
 TIGHT_16 = 2e-5    # what identical operands + fp32 accumulation actually give
+TIGHT_POST = 4e-3  # post-scaled int4: bf16 rounding of the weights is not applied
 
 
 def _check(orc, rng, M, N, K, kind, cd, xd, group=128, yd=0):
@@ -31,7 +35,8 @@ def _check(orc, rng, M, N, K, kind, cd, xd, group=128, yd=0):
     bound = TOL_32 if cd == 0 else TOL_16
     assert err <= bound, (M, N, K, kind, cd, xd, err)
     if cd != 0 and yd == 0:
-        assert err <= TIGHT_16, (M, N, K, kind, cd, xd, err)
+        post = kind == "int4" and group % 128 == 0
+        assert err <= (TIGHT_POST if post else TIGHT_16), (M, N, K, kind, cd, xd, err)
     return err
 
 
@@ -61,7 +66,7 @@ def test_ragged_and_wave_count_variants(orc, N, K, M):
     _check(orc, rng, M, N, K, "int8pc", 2, 2)
 
 
-@pytest.mark.parametrize("group", [32, 64, 256])
+@pytest.mark.parametrize("group", [32, 64, 256, 512])
 def test_int4_group_sizes(orc, group):
     _check(orc, np.random.default_rng(group), 2, 128, 1024, "int4", 2, 2, group=group)
 
@@ -77,16 +82,20 @@ def test_m1_equals_row0_of_m16(orc):
     x = dev_as(rng.normal(0, 1, (16, 2048)), 2)
     y16 = host(T.qlinear_forward(x, dw, 2))
     y1 = host(T.qlinear_forward(x[:1].contiguous(), dw, 2))
-    assert np.array_equal(y16[0], y1[0])
+    y4 = host(T.qlinear_forward(x[:4].contiguous(), dw, 2))
+    # different M take different kernels (summation order differs), so equal up to fp32 rounding
+    assert np.abs(y16[0] - y1[0]).max() <= 1e-5 * np.abs(y16).max()
+    assert np.abs(y16[:4] - y4).max() <= 1e-5 * np.abs(y16).max()
 
 
 def test_one_hot_reads_a_weight_column_exactly(orc):
-    # X = e_j  =>  Y[0, n] = W[n, j] in the compute dtype, exactly (a single non-zero product)
+    # X = e_j  =>  Y[0, n] = W[n, j] exactly (a single non-zero product): in the compute dtype for the
+    # paths that round each weight, as the unrounded fp32 code*scale for post-scaled int4 (group 128)
     rng = np.random.default_rng(6)
-    for kind in ("int4", "int8pc"):
-        ow, dw = make_weight(orc, rng, 320, 1024, kind)
-        for j in (0, 1, 127, 128, 777, 1023):
+    for kind, group, wd in (("int4", 128, 0), ("int4", 64, 2), ("int8pc", 128, 2), ("int8pt", 128, 2)):
+        ow, dw = make_weight(orc, rng, 320, 1024, kind, group)
+        for j in (0, 1, 4, 127, 128, 777, 1023):
             e = np.zeros((1, 1024), np.float32)
             e[0, j] = 1.0
             y = host(T.qlinear_forward(dev_as(e, 2), dw, 2))
-            assert np.array_equal(y[0], ow.compute_weight(2)[:, j]), (kind, j)
+            assert np.array_equal(y[0], ow.compute_weight(wd)[:, j]), (kind, group, j)
