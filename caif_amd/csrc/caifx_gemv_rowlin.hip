@@ -362,7 +362,7 @@ template <typename CT, int MT, int CPR>
 __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
 {
   typedef typename Mfma16<CT>::vec_t vec_t;
-  constexpr int D = 8 / CPR;                 // rows in flight
+  constexpr int D = (CPR >= 4) ? 1 : 4 / CPR;   // rows in flight (measured best: 4 loads per lane)
   constexpr int kPieces = CPR * 256;         // 8-value pieces per activation row
   constexpr int kGroupsPad = CPR * 16;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -378,7 +378,7 @@ __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
   const int di = lane & 15;
   const int pslot = di * 4 + (lane >> 4);
   constexpr int64_t kRowBytes = static_cast<int64_t>(CPR) * 1024;
-  const int groups_per_row = (CPR * 2048) >> a.group_shift;
+  constexpr int groups_per_row = CPR * 16;       // group size 128
 
   XPieces<CT, MT, kPieces> xp;
   x_request<CT, MT, kPieces>(a, xp);
@@ -391,7 +391,7 @@ __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
 #pragma unroll
     for (int c = 0; c < CPR; ++c) {
       w[d][c] = *reinterpret_cast<const u32x4_t *>(wp + r * kRowBytes + c * 1024);
-      sc[d][c] = sp[r * groups_per_row + ((c * 2048 + di * 128) >> a.group_shift)];
+      sc[d][c] = sp[r * groups_per_row + c * 16 + di];
     }
   };
 #pragma unroll
@@ -456,7 +456,7 @@ __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
           const float v = wave_sum_hi(is_diag ? tot[m] : 0.0f);
-          if (lane == 63 && m < a.M) store_y(a.y, a.y_dtype, static_cast<int64_t>(m) * a.N + row0 + r, v);
+          if (lane == 63 && (MT != 4 || m < a.M)) static_cast<float *>(a.y)[static_cast<int64_t>(m) * a.N + row0 + r] = v;
         }
       }
     }
@@ -467,7 +467,7 @@ template <typename CT, int MT, bool kVec, int CPR>
 __global__ __launch_bounds__(256) void rowlin_int8_fast_kernel(RowArgs a)
 {
   typedef typename Mfma16<CT>::vec_t vec_t;
-  constexpr int D = 8 / CPR;                 // rows in flight
+  constexpr int D = (CPR >= 4) ? 1 : 4 / CPR;   // rows in flight
   constexpr int kPieces = CPR * 128;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   CT *xs = reinterpret_cast<CT *>(smem);     // [MT][CPR*1024]
@@ -561,7 +561,7 @@ __global__ __launch_bounds__(256) void rowlin_int8_fast_kernel(RowArgs a)
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
           const float v = wave_sum_hi(diag_of(acc[m], lane));
-          if (lane == 63 && m < a.M) store_y(a.y, a.y_dtype, static_cast<int64_t>(m) * a.N + nrow, v);
+          if (lane == 63 && (MT != 4 || m < a.M)) static_cast<float *>(a.y)[static_cast<int64_t>(m) * a.N + nrow] = v;
         }
       }
     }
@@ -702,7 +702,7 @@ template <typename CT, typename XT, int MT>
 int launch_int4(const RowArgs &ra, hipStream_t s)
 {
   if constexpr (dtype_code<XT>::value == dtype_code<CT>::value) {
-    const bool full = (ra.K % 2048 == 0);
+    const bool full = (ra.K % 2048 == 0) && ra.group_shift == 7 && ra.y_dtype == CAIFX_F32;
     if (full && ra.cpr == 1) return launch_int4_fast<CT, MT, 1>(ra, s);
     if (full && ra.cpr == 2) return launch_int4_fast<CT, MT, 2>(ra, s);
     if (full && ra.cpr == 4) return launch_int4_fast<CT, MT, 4>(ra, s);
@@ -717,7 +717,7 @@ template <typename CT, typename XT, int MT, bool kVec>
 int launch_int8(const RowArgs &ra, hipStream_t s)
 {
   if constexpr (dtype_code<XT>::value == dtype_code<CT>::value) {
-    const bool full = (ra.K % 1024 == 0);
+    const bool full = (ra.K % 1024 == 0) && ra.y_dtype == CAIFX_F32;
     if (full && ra.cpr == 1) return launch_int8_fast<CT, MT, kVec, 1>(ra, s);
     if (full && ra.cpr == 2) return launch_int8_fast<CT, MT, kVec, 2>(ra, s);
     if (full && ra.cpr == 4) return launch_int8_fast<CT, MT, kVec, 4>(ra, s);
