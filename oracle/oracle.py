@@ -344,3 +344,37 @@ def moe_build_dispatch_map(indices, num_experts, capacity_per_expert=0):
     total = lib().orc_moe_build_dispatch_map(_ptr(idx), T, num_experts, top_k, capacity_per_expert,
                                              _ptr(dmap), _ptr(offsets))
     return dmap, offsets, int(total)
+
+
+# --------------------------------------------------------------------------- LoRA around a frozen base
+def lora_forward(x_values, fw, lora_a, lora_b, alpha, compute_dtype, storage_dtype):
+    """CAIF_DeviceLoRAAdapter::ForwardImpl (src/caif_device_lora_adapter.cpp:119-203):
+    base_out = base(x) (fp32, cast to the storage dtype, :189-198); lora_hidden = x A^T and
+    lora_out = lora_hidden B^T are stored in the storage dtype (:161-173); lora_out is scaled by
+    alpha/rank in place (:175-177) and added element-wise (:187-198).  A is [rank, in], B is
+    [out, rank].  Returns (output, lora_hidden)."""
+    x = round_to_dtype(np.asarray(x_values, np.float32), storage_dtype)
+    rank = lora_a.shape[0]
+    base = round_to_dtype(frozen_linear_forward(x, fw, compute_dtype), storage_dtype)
+    a = round_to_dtype(lora_a, storage_dtype)
+    b = round_to_dtype(lora_b, storage_dtype)
+    hidden = round_to_dtype(gemm_nt(x, a), storage_dtype)
+    out = round_to_dtype(gemm_nt(hidden, b), storage_dtype)
+    out = round_to_dtype(out * np.float32(alpha / rank), storage_dtype)
+    return add(base, out, storage_dtype), hidden
+
+
+def lora_backward_input(grad_values, fw, lora_a, lora_b, alpha, compute_dtype, storage_dtype):
+    """Input gradient of CAIF_DeviceLoRAAdapter::BackwardImpl (src/caif_device_lora_adapter.cpp:
+    205-281): d_lora_scaled = g * alpha/rank (:228-232); d_lora_hidden = d_lora_scaled B (:241-243);
+    d_input_lora = d_lora_hidden A (:250-252); grad_base = base.Backward(g) (:255), cast to the
+    storage dtype and added (:267-276)."""
+    g = round_to_dtype(np.asarray(grad_values, np.float32), storage_dtype)
+    rank = lora_a.shape[0]
+    a = round_to_dtype(lora_a, storage_dtype)
+    b = round_to_dtype(lora_b, storage_dtype)
+    gs = round_to_dtype(g * np.float32(alpha / rank), storage_dtype)
+    d_hidden = round_to_dtype(gemm_nn(gs, b), storage_dtype)
+    d_in = round_to_dtype(gemm_nn(d_hidden, a), storage_dtype)
+    base = round_to_dtype(frozen_linear_backward(g, fw, compute_dtype), storage_dtype)
+    return add(base, d_in, storage_dtype)

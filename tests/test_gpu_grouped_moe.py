@@ -1,0 +1,127 @@
+"""GPU parity of the grouped (token-sorted expert segments) dequant-GEMMs and of the frozen SwiGLU
+expert layer built from them, against the CPU oracle's per-expert restatement of
+CAIF_DeviceMoEFrozenExpert (src/caif_device_moe_frozen_expert.cpp:92-332)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from caif_amd import torch_ops as T                                  # noqa: E402
+from gpu_helpers import dev, dev_as, host, make_weight, max_rel_err   # noqa: E402
+
+TOL = 1e-2
+
+
+def _experts(orc, rng, E, N, K, kind, group=128):
+    pairs = [make_weight(orc, rng, N, K, kind, group) for _ in range(E)]
+    return [p[0] for p in pairs], T.GroupedFrozenWeights([p[1] for p in pairs])
+
+
+@pytest.mark.parametrize("kind", ["int8pc", "int4", "int8pt"])
+def test_grouped_forward_backward_segments(orc, kind):
+    rng = np.random.default_rng(1)
+    E, N, K = 6, 192, 256
+    counts = np.array([130, 0, 1, 257, 64, 5])                       # empty, tiny and multi-tile segments
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    total = int(offsets[-1])
+    ows, gw = _experts(orc, rng, E, N, K, kind, group=64)
+    x = dev_as(rng.normal(0, 1, (total + 3, K)), 2)                  # 3 rows past offsets[E]: untouched
+    dy = dev_as(rng.normal(0, 1e-2, (total + 3, N)), 2)
+    off_d = dev(offsets)
+    y = host(T.qlinear_grouped_forward(x, off_d, gw, 2))
+    dx = host(T.qlinear_grouped_backward_input(dy, off_d, gw, 2))
+    xh, dyh = host(x), host(dy)
+    for e in range(E):
+        lo, hi = offsets[e], offsets[e + 1]
+        if hi == lo:
+            continue
+        assert max_rel_err(y[lo:hi], orc.frozen_linear_forward(xh[lo:hi], ows[e], 2)) <= 5e-5
+        assert max_rel_err(dx[lo:hi], orc.frozen_linear_backward(dyh[lo:hi], ows[e], 2)) <= 5e-5
+    assert not y[total:].any() and not dx[total:].any()
+
+
+def test_grouped_equals_per_expert_calls(orc):
+    rng = np.random.default_rng(2)
+    E, N, K = 4, 256, 128
+    counts = np.array([100, 28, 200, 60])
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    ows, gw = _experts(orc, rng, E, N, K, "int8pc")
+    x = dev_as(rng.normal(0, 1, (int(offsets[-1]), K)), 2)
+    y = T.qlinear_grouped_forward(x, dev(offsets), gw, 2, T.BF16)
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        ye = T.qlinear_forward(x[lo:hi].contiguous(), gw.weights[e], 2, T.BF16)
+        if hi - lo > 16:                                             # same kernel family: bit-identical
+            assert torch.equal(y[lo:hi], ye)
+
+
+def _route(rng, Tk, top_k, E):
+    idx = rng.integers(0, E, (Tk, top_k)).astype(np.int32)
+    return idx
+
+
+def test_moe_frozen_expert_layer_forward_backward(orc):
+    """DeepSeek-V2-Lite-like frozen SwiGLU experts at reduced width: int8 per-channel weights, bf16
+    tokens, top-k routing with uniform random expert ids (repeats allowed), forward + backward dX.
+    The segment layout is the reference's dispatch map (token-major arrival order)."""
+    rng = np.random.default_rng(3)
+    E, D, H, Tk, top_k = 8, 256, 192, 96, 3
+    idx = _route(rng, Tk, top_k, E)
+    dmap, offsets, total = orc.moe_build_dispatch_map(idx, E)
+    rows = offsets[idx] + dmap                                       # packed row of assignment (t, k)
+    xt = orc.round_to_dtype(rng.normal(0, 1, (Tk, D)), 2)
+    packed = np.zeros((total, D), np.float32)
+    packed[rows.ravel()] = np.repeat(xt, top_k, axis=0)              # what MoEDispatchGPU packs
+    gate_o, gate_g = _experts(orc, rng, E, H, D, "int8pc")
+    up_o, up_g = _experts(orc, rng, E, H, D, "int8pc")
+    down_o, down_g = _experts(orc, rng, E, D, H, "int8pc")
+    gout = orc.round_to_dtype(rng.normal(0, 1e-2, (total, D)), 2)
+
+    off_d = dev(offsets)
+    x = dev_as(packed, 2)
+    # forward: each frozen linear's fp32 output is rounded to bf16 in the GEMM's store
+    up_out = T.qlinear_grouped_forward(x, off_d, up_g, T.BF16, T.BF16)
+    gate_out = T.qlinear_grouped_forward(x, off_d, gate_g, T.BF16, T.BF16)
+    hidden = T.silu_multiply(gate_out, up_out)
+    out = T.qlinear_grouped_forward(hidden, off_d, down_g, T.BF16, T.BF16)
+    # backward
+    g = dev_as(gout, 2)
+    grad_hidden = T.qlinear_grouped_backward_input(g, off_d, down_g, T.BF16, T.BF16)
+    gate_act = T.silu(gate_out)
+    grad_up = T.multiply(grad_hidden, gate_act)
+    grad_gate = T.silu_backward(gate_out, T.multiply(grad_hidden, up_out))
+    gi_up = T.qlinear_grouped_backward_input(grad_up, off_d, up_g, T.BF16, T.BF16)
+    gi_gate = T.qlinear_grouped_backward_input(grad_gate, off_d, gate_g, T.BF16, T.BF16)
+    dx = T.add(gi_up, gi_gate)
+
+    outh, dxh, hidh = host(out), host(dx), host(hidden)
+    for e in range(E):
+        lo, hi = offsets[e], offsets[e + 1]
+        if hi == lo:
+            continue
+        want, cache = orc.moe_frozen_expert_forward(packed[lo:hi], gate_o[e], up_o[e], down_o[e], 2, 2)
+        # intermediate bf16 roundings can flip by one ulp where the fp32 sums differ in the last bit
+        assert max_rel_err(hidh[lo:hi], cache["hidden"]) <= TOL
+        assert max_rel_err(outh[lo:hi], want) <= TOL
+        wdx = orc.moe_frozen_expert_backward(gout[lo:hi], cache, gate_o[e], up_o[e], down_o[e], 2, 2)
+        assert max_rel_err(dxh[lo:hi], wdx) <= TOL
+
+
+def test_elementwise_ops_match_oracle(orc):
+    rng = np.random.default_rng(4)
+    n = 8 * 1000 + 5                                                 # vector body + scalar tail
+    a = rng.normal(0, 2, n).astype(np.float32)
+    b = rng.normal(0, 2, n).astype(np.float32)
+    for dt, tol in ((0, 2e-6), (2, 0.0), (1, 0.0)):
+        ad, bd = dev_as(a, dt), dev_as(b, dt)
+        ah, bh = host(ad), host(bd)
+        # expf differs by a few ulp between libm and the device: allow one ulp of the tensor dtype
+        ulp = {0: 2e-6, 1: 2 ** -10, 2: 2 ** -7}[dt]
+        for got, want in ((T.silu(ad), orc.silu(ah, dt)),
+                          (T.silu_backward(ad, bd), orc.silu_backward(ah, bh, dt)),
+                          (T.silu_multiply(ad, bd), orc.multiply(orc.silu(ah, dt), bh, dt))):
+            g, w = host(got), want
+            assert np.all(np.abs(g - w) <= ulp * np.maximum(np.abs(w), 1e-3) * 1.01)
+        assert np.array_equal(host(T.multiply(ad, bd)), orc.multiply(ah, bh, dt))   # exact
+        assert np.array_equal(host(T.add(ad, bd)), orc.add(ah, bh, dt))             # exact
