@@ -27,6 +27,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 K_DEC, N_DEC = 4096, 14336
+MEASURED_TRAFFIC_INT8_M1 = 59798477     # bytes per launch, rocprofv3 counters (see the roofline object)
 
 
 def algorithmic_bytes(kind, M, N=N_DEC, K=K_DEC, group=128):
@@ -45,6 +46,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary rows (M=4/16, GEMM TFLOP/s)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy three times (reference point for rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
@@ -126,6 +130,14 @@ def main():
     step_bytes = algorithmic_bytes("int4", 1) + algorithmic_bytes("int8", 1)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    if args.calibrate_copy:
+        src = torch.empty(256 * 2**20, dtype=torch.uint8, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---------------------------------------------------------------- per-kernel durations (HIP events)
     L = 64
     per = {}
@@ -147,14 +159,17 @@ def main():
     dom = ("int8", 1)           # the kernel that takes most of a step
     roofline = {
         "bound": "hbm",
-        "kernel": "skinny_forward_kernel<bf16,bf16,int8 per-channel> M=1 K=4096 N=14336",
+        "kernel": "rowlin_int8_fast_kernel<bf16, 1 row, per-channel scales, 4 chunks/row> M=1 K=4096 N=14336",
         "achieved": round(per[dom]["GBps"], 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(per[dom]["GBps"] / HBM_PEAK_GBS, 4),
         "avg_launch_us": round(per[dom]["us"], 3),
         "algorithmic_bytes_per_launch": algorithmic_bytes("int8", 1),
-        "traffic": None,
+        # HBM bytes per launch of this kernel from two rocprofv3 --pmc runs (FETCH_SIZE x 1.9998 and
+        # WRITE_SIZE x 1.0000, factors from a plain 256 MiB copy in the same runs): 59.36 MB read +
+        # 0.44 MB written; the summary is profiles/decode_gemv_hbm_traffic.md
+        "traffic": MEASURED_TRAFFIC_INT8_M1,
     }
 
     extra = {
