@@ -6,27 +6,29 @@
 // with B drawn from the stored weight W[N,K]:
 //     forward : C = N, R = K, B[r][c] = W[c][r]   (a weight row is contiguous along R)
 //     backward: C = K, R = N, B[r][c] = W[r][c]   (a weight row is contiguous along C)
-// A workgroup (256 threads, 2x2 waves) owns a 128 x 128 tile of D and walks R in steps of 64.
-// Per step it moves a 128x64 tile of A and the matching 64x128 piece of W from global memory
-// into registers while the matrix cores work on the previous step, then dequantises W in
+// A workgroup (256 threads, 2x2 waves) owns a BM x 128 tile of D (BM = 128 is what is launched)
+// and walks R in steps of 64.
+// Per step it moves a BMx64 tile of A and the matching 64x128 piece of W from global memory
+// into registers two steps ahead of their use, dequantises W in
 // registers (code * scale in fp32, one rounding to the compute dtype: bit-identical to the
 // reference's dequantise-then-cast weight) and writes both tiles to the other half of a
 // double-buffered LDS area, as [row][64 values along R] with the 16-byte chunks of a row
 // XOR-swizzled by (row & 7) so that the 128-bit operand reads of v_mfma_f32_32x32x16 spread
 // over all banks.  For the backward case the weight piece is transposed on the way: a thread
 // holds 4 weight rows x 8 columns and writes 8 runs of 4 values along R.
-// Each wave accumulates a 64 x 64 sub-tile (2x2 MFMA tiles, 64 fp32 accumulators per lane).
+// Each wave accumulates a (BM/2) x 64 sub-tile (64 or 128 fp32 accumulators per lane).
 // No dense copy of W ever reaches HBM; the only HBM traffic is A, the packed W and D.
 #include "caifx_internal.hpp"
+
+#include <type_traits>
 
 namespace caifx {
 namespace {
 
-constexpr int BM = 128;      // rows of D per workgroup
 constexpr int BC = 128;      // columns of D per workgroup
 constexpr int BR = 64;       // reduction extent per step
 constexpr int kThreads = 256;
-constexpr int kTileBytes = 128 * BR * 2;   // one operand tile in LDS (16 KiB)
+constexpr int kBTileBytes = BC * BR * 2;   // weight tile in LDS (16 KiB)
 
 template <typename CT> struct Mfma32;
 template <> struct Mfma32<bf16_t> {
@@ -63,8 +65,10 @@ struct TileArgs {
   int num_experts;
 };
 
-// byte offset of 16-byte chunk `chunk` (0..7) of LDS tile row `row`
-__device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
+// byte offset of 16-byte chunk `chunk` (0..7) of LDS tile row `row`.  The chunk position is XORed
+// with bits of the row so that (a) 8 consecutive rows at one chunk index and (b) rows 8 apart at one
+// chunk index (the transposed weight writes of the backward case) land in different banks.
+__device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + ((chunk ^ ((row ^ (row >> 3)) & 7)) << 4); }
 
 template <typename CT> __device__ __forceinline__ uint32_t pack2(float lo, float hi)
 {
@@ -81,15 +85,20 @@ __device__ __forceinline__ float int8_scale_at(const float *scales, int mode, in
   return scales[flat % period];
 }
 
-template <typename CT, typename XT, bool kInt4, bool kBackward, bool kGrouped>
+// BM: rows of D per workgroup (128 or 256); a wave owns (BM/2) x 64 of D.
+template <typename CT, typename XT, bool kInt4, bool kBackward, bool kGrouped, int BM>
 __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
 {
   typedef typename Mfma32<CT>::vec_t vec_t;
-  __shared__ __attribute__((aligned(16))) unsigned char smem[4 * kTileBytes];   // A0 B0 A1 B1
+  constexpr int kATileBytes = BM * BR * 2;
+  constexpr int kStageBytes = kATileBytes + kBTileBytes;     // one buffer: A tile then B tile
+  constexpr int WR = BM / 64;                                // 32-row MFMA tiles per wave along M
+  constexpr int kAChunks = BM / 32;                          // 16-byte LDS chunks of A per thread per step
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];          // 2 x kStageBytes
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1;      // wave row (0..1): 64 rows of D
+  const int wm = wave >> 1;      // wave row (0..1): BM/2 rows of D
   const int wc = wave & 1;       // wave column (0..1): 64 columns of D
 
   const int64_t R = kBackward ? g.N : g.K;     // reduction length
@@ -128,46 +137,53 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
   const XT *ag = static_cast<const XT *>(g.a);
 
   // ---- global -> register staging ---------------------------------------------------------
-  // A tile: 128 rows x 8 chunks (8 values each); thread handles chunks q = tid + 256*i, i < 4
-  constexpr int kAVecs = (sizeof(XT) == 4) ? 8 : 4;     // 16-byte loads per thread per step
-  u32x4_t areg[kAVecs];
-  int a_row[4], a_chunk[4];
-  const XT *a_ptr[4];
+  // Two register sets: while the matrix cores work on the tile in LDS buffer (s & 1), set (s+1)&1
+  // (loaded one step earlier) is dequantised into the other buffer and set s&1 receives tile s+2
+  // from global memory.  (A third set, i.e. two steps of load latency, measured no faster.)  The store work is cut in four parts, one per 16-wide k step, so that it
+  // can be interleaved with the MFMAs of that k step.
+  // A tile: BM rows x 8 chunks (8 values each); thread handles chunks q = tid + 256*i
+  constexpr int kAVecs = (sizeof(XT) == 4) ? 2 * kAChunks : kAChunks;     // 16-byte loads per thread per step
+  u32x4_t areg[2][kAVecs];
+  int a_off[kAChunks];            // LDS byte offset of each chunk inside the A tile
+  const XT *a_ptr[kAChunks];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < kAChunks; ++i) {
     const int q = tid + kThreads * i;
-    a_row[i] = q >> 3;
-    a_chunk[i] = q & 7;
-    int64_t m = row_lo + a_row[i];
+    a_off[i] = swz(q >> 3, q & 7);
+    int64_t m = row_lo + (q >> 3);
     if (m >= row_hi) m = row_hi - 1;                    // clamp: rows past the end are never stored
-    a_ptr[i] = ag + m * R + a_chunk[i] * 8;
+    a_ptr[i] = ag + m * R + (q & 7) * 8;
   }
-  auto load_a = [&](int64_t r0) {
+  auto load_a = [&](auto set_, int64_t r0) {
+    constexpr int set = decltype(set_)::value;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kAChunks; ++i) {
       if constexpr (sizeof(XT) == 4) {
-        areg[2 * i] = *reinterpret_cast<const u32x4_t *>(a_ptr[i] + r0);
-        areg[2 * i + 1] = *reinterpret_cast<const u32x4_t *>(a_ptr[i] + r0 + 4);
+        areg[set][2 * i] = *reinterpret_cast<const u32x4_t *>(a_ptr[i] + r0);
+        areg[set][2 * i + 1] = *reinterpret_cast<const u32x4_t *>(a_ptr[i] + r0 + 4);
       } else {
-        areg[i] = *reinterpret_cast<const u32x4_t *>(a_ptr[i] + r0);
+        areg[set][i] = *reinterpret_cast<const u32x4_t *>(a_ptr[i] + r0);
       }
     }
   };
-  auto store_a = [&](unsigned char *dst) {
+  auto store_a = [&](auto set_, unsigned char *dst, int part) {
+    constexpr int set = decltype(set_)::value;
+    constexpr int per = kAChunks / 4;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int ii = 0; ii < per; ++ii) {
+      const int i = part * per + ii;
       u32x4_t v;
       if constexpr (sizeof(XT) == 4) {
-        const float *f0 = reinterpret_cast<const float *>(&areg[2 * i]);
-        const float *f1 = reinterpret_cast<const float *>(&areg[2 * i + 1]);
+        const float *f0 = reinterpret_cast<const float *>(&areg[set][2 * i]);
+        const float *f1 = reinterpret_cast<const float *>(&areg[set][2 * i + 1]);
         v[0] = pack2<CT>(f0[0], f0[1]);
         v[1] = pack2<CT>(f0[2], f0[3]);
         v[2] = pack2<CT>(f1[0], f1[1]);
         v[3] = pack2<CT>(f1[2], f1[3]);
       } else {
-        v = areg[i];
+        v = areg[set][i];
       }
-      *reinterpret_cast<u32x4_t *>(dst + swz(a_row[i], a_chunk[i])) = v;
+      *reinterpret_cast<u32x4_t *>(dst + a_off[i]) = v;
     }
   };
 
@@ -176,8 +192,8 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
   //   forward  int8: rows c = tid/4 (+64), 16 codes (16 B) at r = (tid%4)*16    -> 2 x 2 chunks
   //   backward int4: rows r = (tid/16)*4 .. +3, 8 codes (4 B) at c = (tid%16)*8 -> 8 runs of 4
   //   backward int8: same rows, 8 codes (8 B)
-  u32x4_t wreg[2];
-  f16_t wscale[4];
+  uint32_t wreg[2][8];
+  f16_t wscale[2][4];
   int64_t w_flat[4];       // flat index n*K + k of each register row's first code at step 0
   const f16_t *s16 = static_cast<const f16_t *>(scales);
   const float *s32 = static_cast<const float *>(scales);
@@ -207,27 +223,34 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
 #pragma unroll
     for (int i = 0; i < 4; ++i) w_flat[i] = static_cast<int64_t>(wf_r + i) * g.K + k;
   }
-  auto load_w = [&](int64_t r0) {
+  auto load_w = [&](auto set_, int64_t r0) {
+    constexpr int set = decltype(set_)::value;
     if constexpr (!kBackward) {
       if constexpr (kInt4) {
         const int64_t f = w_flat[0] + r0;
-        wreg[0] = *reinterpret_cast<const u32x4_t *>(wq + (f >> 1));
-        wscale[0] = s16[f >> g.group_shift];
+        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(wq + (f >> 1));
+#pragma unroll
+        for (int j = 0; j < 4; ++j) wreg[set][j] = v[j];
+        wscale[set][0] = s16[f >> g.group_shift];
       } else {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) wreg[i] = *reinterpret_cast<const u32x4_t *>(wq + w_flat[i] + r0);
+        for (int i = 0; i < 2; ++i) {
+          const u32x4_t v = *reinterpret_cast<const u32x4_t *>(wq + w_flat[i] + r0);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) wreg[set][4 * i + j] = v[j];
+        }
       }
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int64_t f = w_flat[i] + r0 * g.K;
         if constexpr (kInt4) {
-          reinterpret_cast<uint32_t *>(wreg)[i] = *reinterpret_cast<const uint32_t *>(wq + (f >> 1));
-          wscale[i] = s16[f >> g.group_shift];
+          wreg[set][i] = *reinterpret_cast<const uint32_t *>(wq + (f >> 1));
+          wscale[set][i] = s16[f >> g.group_shift];
         } else {
           const u32x2_t v = *reinterpret_cast<const u32x2_t *>(wq + f);
-          reinterpret_cast<uint32_t *>(wreg)[2 * i] = v[0];
-          reinterpret_cast<uint32_t *>(wreg)[2 * i + 1] = v[1];
+          wreg[set][2 * i] = v[0];
+          wreg[set][2 * i + 1] = v[1];
         }
       }
     }
@@ -245,124 +268,159 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
       for (int j = 0; j < 4; ++j) out[j] = q[j] * int8_scale_at(s32, g.scale_mode, g.period, f + j);
     }
   };
-  auto store_w = [&](unsigned char *dst, int64_t r0) {
+  // Backward keeps the dequantised 4 x 8 block between parts: parts 0..3 dequantise one weight row
+  // each, part 3 then writes the 8 transposed runs.
+  float et[4][8];
+  auto store_w = [&](auto set_, unsigned char *dst, int64_t r0, int part) {
+    constexpr int set = decltype(set_)::value;
     if constexpr (!kBackward) {
       if constexpr (kInt4) {
-        const float s = to_f32(wscale[0]);
+        const float s = to_f32(wscale[set][0]);
+        const int j = part;
+        float e[8];
+        dequant_int4x8(wreg[set][j], s, e);
+        u32x4_t v;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float e[8];
-          dequant_int4x8(wreg[0][j], s, e);
-          u32x4_t v;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) v[q] = pack2<CT>(e[2 * q], e[2 * q + 1]);
-          *reinterpret_cast<u32x4_t *>(dst + swz(wf_c, (wf_r >> 3) + j)) = v;
-        }
+        for (int q = 0; q < 4; ++q) v[q] = pack2<CT>(e[2 * q], e[2 * q + 1]);
+        *reinterpret_cast<u32x4_t *>(dst + swz(wf_c, (wf_r >> 3) + j)) = v;
       } else {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            float lo[4], hi[4];
-            deq8(wreg[i][2 * j], w_flat[i] + r0 + 8 * j, lo);
-            deq8(wreg[i][2 * j + 1], w_flat[i] + r0 + 8 * j + 4, hi);
-            u32x4_t v;
-            v[0] = pack2<CT>(lo[0], lo[1]);
-            v[1] = pack2<CT>(lo[2], lo[3]);
-            v[2] = pack2<CT>(hi[0], hi[1]);
-            v[3] = pack2<CT>(hi[2], hi[3]);
-            *reinterpret_cast<u32x4_t *>(dst + swz(wf_c + 64 * i, (wf_r >> 3) + j)) = v;
-          }
-        }
+        const int i = part >> 1;
+        const int j = part & 1;
+        float lo[4], hi[4];
+        deq8(wreg[set][4 * i + 2 * j], w_flat[i] + r0 + 8 * j, lo);
+        deq8(wreg[set][4 * i + 2 * j + 1], w_flat[i] + r0 + 8 * j + 4, hi);
+        u32x4_t v;
+        v[0] = pack2<CT>(lo[0], lo[1]);
+        v[1] = pack2<CT>(lo[2], lo[3]);
+        v[2] = pack2<CT>(hi[0], hi[1]);
+        v[3] = pack2<CT>(hi[2], hi[3]);
+        *reinterpret_cast<u32x4_t *>(dst + swz(wf_c + 64 * i, (wf_r >> 3) + j)) = v;
       }
     } else {
-      // e[i][j]: weight row (reduction index) wf_r + i, column wf_c + j
-      float e[4][8];
+      const int i = part;      // et[i][j]: weight row (reduction index) wf_r + i, column wf_c + j
+      if constexpr (kInt4) {
+        dequant_int4x8(wreg[set][i], to_f32(wscale[set][i]), et[i]);
+      } else {
+        const int64_t f = w_flat[i] + r0 * g.K;
+        float lo[4], hi[4];
+        deq8(wreg[set][2 * i], f, lo);
+        deq8(wreg[set][2 * i + 1], f + 4, hi);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if constexpr (kInt4) {
-          dequant_int4x8(reinterpret_cast<const uint32_t *>(wreg)[i], to_f32(wscale[i]), e[i]);
-        } else {
-          const int64_t f = w_flat[i] + r0 * g.K;
-          float lo[4], hi[4];
-          deq8(reinterpret_cast<const uint32_t *>(wreg)[2 * i], f, lo);
-          deq8(reinterpret_cast<const uint32_t *>(wreg)[2 * i + 1], f + 4, hi);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            e[i][j] = lo[j];
-            e[i][4 + j] = hi[j];
-          }
+        for (int j = 0; j < 4; ++j) {
+          et[i][j] = lo[j];
+          et[i][4 + j] = hi[j];
         }
       }
-      // transposed write: LDS row = column c, run of 4 values along R at r = wf_r .. wf_r+3
+      if (part == 3) {
+        // transposed write: LDS row = column c, run of 4 values along R at r = wf_r .. wf_r+3
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        u32x2_t v;
-        v[0] = pack2<CT>(e[0][j], e[1][j]);
-        v[1] = pack2<CT>(e[2][j], e[3][j]);
-        const int row = wf_c + j;
-        *reinterpret_cast<u32x2_t *>(dst + swz(row, wf_r >> 3) + ((wf_r & 4) << 1)) = v;
+        for (int j = 0; j < 8; ++j) {
+          u32x2_t v;
+          v[0] = pack2<CT>(et[0][j], et[1][j]);
+          v[1] = pack2<CT>(et[2][j], et[3][j]);
+          *reinterpret_cast<u32x2_t *>(dst + swz(wf_c + j, wf_r >> 3) + ((wf_r & 4) << 1)) = v;
+        }
       }
     }
   };
 
   // ---- main loop ------------------------------------------------------------------------
-  floatx16_t acc[2][2];
+  floatx16_t acc[WR][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WR; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   const int steps = static_cast<int>(R / BR);
-  load_a(0);
-  load_w(0);
-  store_a(smem);
-  store_w(smem + kTileBytes, 0);
+  const int last = steps - 1;
+  typedef std::integral_constant<int, 0> I0;
+  typedef std::integral_constant<int, 1> I1;
+  auto tile_r0 = [&](int t) { return static_cast<int64_t>(t < last ? t : last) * BR; };   // clamped: reloading the last tile is harmless
+
+  load_a(I0{}, 0);
+  load_w(I0{}, 0);
+#pragma unroll
+  for (int part = 0; part < 4; ++part) {
+    store_a(I0{}, smem, part);
+    store_w(I0{}, smem + kATileBytes, 0, part);
+  }
+  load_a(I1{}, tile_r0(1));
+  load_w(I1{}, tile_r0(1));
   __syncthreads();
 
   const int frow = lane & 31;    // row of the operand tile this lane supplies
   const int fh = lane >> 5;      // which half of the 16-wide k step
-  for (int s = 0; s < steps; ++s) {
-    const unsigned char *abuf = smem + (s & 1) * 2 * kTileBytes;
-    const unsigned char *bbuf = abuf + kTileBytes;
-    const bool more = (s + 1 < steps);
-    if (more) {
-      load_a(static_cast<int64_t>(s + 1) * BR);
-      load_w(static_cast<int64_t>(s + 1) * BR);
-    }
+  int a_frag_off[WR], b_frag_off[2];   // LDS byte offsets of this lane's operand rows (chunk 0, before the swizzle)
+  // One step s: MFMAs on LDS buffer `buf` (= s & 1); the tile held in the other register set goes
+  // to the other buffer; register set `buf` is refilled with tile s+2.
+  auto step = [&](auto buf_, int s) {
+    constexpr int buf = decltype(buf_)::value;
+    typedef decltype(buf_) CurSet;
+    typedef std::integral_constant<int, 1 - buf> NxtSet;
+    const unsigned char *abuf = smem + buf * kStageBytes;
+    const unsigned char *bbuf = abuf + kATileBytes;
+    unsigned char *nbuf = smem + (1 - buf) * kStageBytes;
+    const int64_t r_next = tile_r0(s + 1);
+    load_a(CurSet{}, tile_r0(s + 2));
+    load_w(CurSet{}, tile_r0(s + 2));
+    // operand fragments are double buffered in registers: the reads of k step ks+1 are issued
+    // before the MFMAs of k step ks
+    vec_t af[2][WR], bf[2][2];
+    auto read_frags = [&](int fb, int ks) {
+#pragma unroll
+      for (int i = 0; i < WR; ++i)
+        af[fb][i] = *reinterpret_cast<const vec_t *>(abuf + swz(wm * (BM / 2) + i * 32 + frow, ks * 2 + fh));
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        bf[fb][j] = *reinterpret_cast<const vec_t *>(bbuf + swz(wc * 64 + j * 32 + frow, ks * 2 + fh));
+    };
+    read_frags(0, 0);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < BR / 16; ++ks) {
-      vec_t af[2], bf[2];
+      const int fsel = ks & 1;
+      if (ks + 1 < BR / 16) read_frags((ks + 1) & 1, ks + 1);
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        af[i] = *reinterpret_cast<const vec_t *>(abuf + swz(wm * 64 + i * 32 + frow, ks * 2 + fh));
-        bf[i] = *reinterpret_cast<const vec_t *>(bbuf + swz(wc * 64 + i * 32 + frow, ks * 2 + fh));
+      for (int i = 0; i < WR; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = Mfma32<CT>::run(af[fsel][i], bf[fsel][j], acc[i][j]);
+      store_a(NxtSet{}, nbuf, ks);
+      store_w(NxtSet{}, nbuf + kATileBytes, r_next, ks);
+      // Order inside the k step: next fragments' reads first, then every MFMA followed by a few
+      // VALU instructions of the dequantisation (one wave has to keep the matrix pipe and the VALU
+      // busy at the same time), LDS writes last.
+      if (ks + 1 < BR / 16) __builtin_amdgcn_sched_group_barrier(0x100, WR + 2, 0);
+#pragma unroll
+      for (int t = 0; t < WR * 2; ++t) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, kBackward ? 8 : 6, 0);
       }
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = Mfma32<CT>::run(af[i], bf[j], acc[i][j]);
-    }
-    if (more) {
-      unsigned char *nbuf = smem + ((s + 1) & 1) * 2 * kTileBytes;
-      store_a(nbuf);
-      store_w(nbuf + kTileBytes, static_cast<int64_t>(s + 1) * BR);
+      __builtin_amdgcn_sched_group_barrier(0x200, 16, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
+  };
+  (void)a_frag_off;
+  (void)b_frag_off;
+  int s = 0;
+  for (; s + 2 <= steps; s += 2) {
+    step(I0{}, s);
+    step(I1{}, s + 1);
   }
+  if (s < steps) step(I0{}, s);
 
   // ---- epilogue: acc[i][j][r] = D[row][col], row = 8*(r/4) + 4*(lane/32) + r%4, col = lane%32
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < WR; ++i) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int64_t col = col0 + wc * 64 + j * 32 + (lane & 31);
       if (col < C) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int64_t row = row_lo + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          const int64_t row = row_lo + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
           if (row < row_hi) {
             const int64_t o = row * C + col;
             const float v = acc[i][j][r];
@@ -376,21 +434,44 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
   }
 }
 
-template <typename CT, typename XT, bool kInt4, bool kBackward>
-int launch_tile(const TileArgs &t, bool grouped, int64_t max_row_tiles, hipStream_t s)
+template <typename CT, typename XT, bool kInt4, bool kBackward, bool kGrouped, int BM>
+int launch_one(const TileArgs &t, int64_t row_tiles, hipStream_t s)
 {
   const int64_t C = kBackward ? t.K : t.N;
-  dim3 grid(static_cast<unsigned>((C + BC - 1) / BC), static_cast<unsigned>(max_row_tiles));
-  if (grouped) hipLaunchKernelGGL((qgemm_kernel<CT, XT, kInt4, kBackward, true>), grid, dim3(kThreads), 0, s, t);
-  else hipLaunchKernelGGL((qgemm_kernel<CT, XT, kInt4, kBackward, false>), grid, dim3(kThreads), 0, s, t);
+  constexpr size_t lds = 2 * (static_cast<size_t>(BM) * BR * 2 + kBTileBytes);
+  auto kern = qgemm_kernel<CT, XT, kInt4, kBackward, kGrouped, BM>;
+  if (lds > 64 * 1024) {
+    static bool raised = false;
+    if (!raised) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(lds)) != hipSuccess)
+        return CAIFX_ERR_LAUNCH_FAILED;
+      raised = true;
+    }
+  }
+  dim3 grid(static_cast<unsigned>((C + BC - 1) / BC), static_cast<unsigned>(row_tiles));
+  hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds, s, t);
   return launch_status();
 }
 
-template <typename CT, typename XT>
-int pick_kind(const TileArgs &t, bool int4, bool backward, bool grouped, int64_t tiles, hipStream_t s)
+// 128-row tiles everywhere: measured on MI355X, two or three resident workgroups per CU (64 KiB of
+// LDS and about 180 registers each) overlap one workgroup's dequantisation with another's MFMAs and
+// reach 1.4-1.9 PFLOP/s, while 256-row tiles (one workgroup per CU) stay near 0.75 PFLOP/s even
+// though they halve the dequantisation work per flop.
+template <typename CT, typename XT, bool kInt4, bool kBackward>
+int launch_tile(const TileArgs &t, bool grouped, hipStream_t s)
 {
-  if (int4) return backward ? launch_tile<CT, XT, true, true>(t, grouped, tiles, s) : launch_tile<CT, XT, true, false>(t, grouped, tiles, s);
-  return backward ? launch_tile<CT, XT, false, true>(t, grouped, tiles, s) : launch_tile<CT, XT, false, false>(t, grouped, tiles, s);
+  const int64_t row_tiles = (t.M + 127) / 128 + (grouped ? t.num_experts : 0);   // every expert can add one partial tile
+  if (row_tiles > 65535) return CAIFX_ERR_UNSUPPORTED;
+  if (grouped) return launch_one<CT, XT, kInt4, kBackward, true, 128>(t, row_tiles, s);
+  return launch_one<CT, XT, kInt4, kBackward, false, 128>(t, row_tiles, s);
+}
+
+template <typename CT, typename XT>
+int pick_kind(const TileArgs &t, bool int4, bool backward, bool grouped, hipStream_t s)
+{
+  if (int4) return backward ? launch_tile<CT, XT, true, true>(t, grouped, s) : launch_tile<CT, XT, true, false>(t, grouped, s);
+  return backward ? launch_tile<CT, XT, false, true>(t, grouped, s) : launch_tile<CT, XT, false, false>(t, grouped, s);
 }
 
 int run(const GemmArgs &a, bool backward, hipStream_t s)
@@ -434,15 +515,12 @@ int run(const GemmArgs &a, bool backward, hipStream_t s)
       t.scale_mode = SM_ANY;
     }
   }
-  // grouped: every expert can add one partial row tile on top of the dense count
-  const int64_t row_tiles = grouped ? (a.M + BM - 1) / BM + a.num_experts : (a.M + BM - 1) / BM;
-  if (row_tiles > 65535) return CAIFX_ERR_UNSUPPORTED;
   if (a.compute_dtype == CAIFX_BF16) {
-    if (a.x_dtype == CAIFX_F32) return pick_kind<bf16_t, float>(t, int4, backward, grouped, row_tiles, s);
-    return pick_kind<bf16_t, bf16_t>(t, int4, backward, grouped, row_tiles, s);
+    if (a.x_dtype == CAIFX_F32) return pick_kind<bf16_t, float>(t, int4, backward, grouped, s);
+    return pick_kind<bf16_t, bf16_t>(t, int4, backward, grouped, s);
   }
-  if (a.x_dtype == CAIFX_F32) return pick_kind<f16_t, float>(t, int4, backward, grouped, row_tiles, s);
-  return pick_kind<f16_t, f16_t>(t, int4, backward, grouped, row_tiles, s);
+  if (a.x_dtype == CAIFX_F32) return pick_kind<f16_t, float>(t, int4, backward, grouped, s);
+  return pick_kind<f16_t, f16_t>(t, int4, backward, grouped, s);
 }
 
 }  // namespace
