@@ -6,8 +6,8 @@
 // with B drawn from the stored weight W[N,K]:
 //     forward : C = N, R = K, B[r][c] = W[c][r]   (a weight row is contiguous along R)
 //     backward: C = K, R = N, B[r][c] = W[r][c]   (a weight row is contiguous along C)
-// A workgroup (256 threads, 2x2 waves) owns a BM x 128 tile of D (BM = 128 is what is launched)
-// and walks R in steps of 64.
+// A workgroup (512 threads: 2x2 consumer waves that run the MFMAs + 4 producer waves that stage the
+// operands) owns a BM x 128 tile of D (BM = 128 is what is launched) and walks R in steps of 64.
 // Per step it moves a BMx64 tile of A and the matching 64x128 piece of W from global memory
 // into registers two steps ahead of their use, dequantises W in
 // registers (code * scale in fp32, one rounding to the compute dtype: bit-identical to the
@@ -27,7 +27,8 @@ namespace {
 
 constexpr int BC = 128;      // columns of D per workgroup
 constexpr int BR = 64;       // reduction extent per step
-constexpr int kThreads = 256;
+constexpr int kStagers = 256;               // producer threads (stage A and W tiles into LDS)
+constexpr int kThreads = 512;               // 4 consumer waves (MFMA) + 4 producer waves
 constexpr int kBTileBytes = BC * BR * 2;   // weight tile in LDS (16 KiB)
 
 template <typename CT> struct Mfma32;
@@ -58,6 +59,7 @@ struct TileArgs {
   int group_shift;           // int4: log2(group_size)
   int scale_mode;            // int8
   int64_t period;            // int8
+  uint32_t scale_step;       // int8, SM_VEC4: how far the scale index moves per 64-deep step, modulo period
   // grouped form
   const int32_t *offsets;
   const void *const *wq_ptrs;
@@ -91,15 +93,17 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
 {
   typedef typename Mfma32<CT>::vec_t vec_t;
   constexpr int kATileBytes = BM * BR * 2;
-  constexpr int kStageBytes = kATileBytes + kBTileBytes;     // one buffer: A tile then B tile
+  constexpr int kAStages = 2;
+  constexpr int kBBase = kAStages * kATileBytes;             // LDS: A ring, then two B buffers
   constexpr int WR = BM / 64;                                // 32-row MFMA tiles per wave along M
   constexpr int kAChunks = BM / 32;                          // 16-byte LDS chunks of A per thread per step
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];          // 2 x kStageBytes
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1;      // wave row (0..1): BM/2 rows of D
-  const int wc = wave & 1;       // wave column (0..1): 64 columns of D
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool producer = wave >= 4;                 // waves 4..7 stage tiles, waves 0..3 run the MFMAs
+  const int tid = threadIdx.x & (kStagers - 1);    // staging thread index (producers)
+  const int wm = (wave >> 1) & 1;  // consumer wave row (0..1): BM/2 rows of D
+  const int wc = wave & 1;         // consumer wave column (0..1): 64 columns of D
 
   const int64_t R = kBackward ? g.N : g.K;     // reduction length
   const int64_t C = kBackward ? g.K : g.N;     // columns of D
@@ -141,14 +145,14 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
   // (loaded one step earlier) is dequantised into the other buffer and set s&1 receives tile s+2
   // from global memory.  (A third set, i.e. two steps of load latency, measured no faster.)  The store work is cut in four parts, one per 16-wide k step, so that it
   // can be interleaved with the MFMAs of that k step.
-  // A tile: BM rows x 8 chunks (8 values each); thread handles chunks q = tid + 256*i
+  // A tile: BM rows x 8 chunks (8 values each); producer thread handles chunks q = tid + 256*i
   constexpr int kAVecs = (sizeof(XT) == 4) ? 2 * kAChunks : kAChunks;     // 16-byte loads per thread per step
   u32x4_t areg[2][kAVecs];
   int a_off[kAChunks];            // LDS byte offset of each chunk inside the A tile
   const XT *a_ptr[kAChunks];
 #pragma unroll
   for (int i = 0; i < kAChunks; ++i) {
-    const int q = tid + kThreads * i;
+    const int q = tid + kStagers * i;
     a_off[i] = swz(q >> 3, q & 7);
     int64_t m = row_lo + (q >> 3);
     if (m >= row_hi) m = row_hi - 1;                    // clamp: rows past the end are never stored
@@ -223,8 +227,43 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
 #pragma unroll
     for (int i = 0; i < 4; ++i) w_flat[i] = static_cast<int64_t>(wf_r + i) * g.K + k;
   }
-  auto load_w = [&](auto set_, int64_t r0) {
+  // int8 with a periodic scale vector (SM_VEC4): the four scales of every code dword travel with
+  // the codes, fetched at position (flat index mod period).  That position is kept per register
+  // row and moved by scale_step after each tile, so no division runs in the loop.
+  floatx4_t wsc8[2][8];
+  uint32_t sidx[4] = {0, 0, 0, 0};
+  const uint32_t period32 = static_cast<uint32_t>(g.period);
+  if constexpr (!kInt4) {
+    if (g.scale_mode == SM_VEC4) {
+#pragma unroll
+      for (int i = 0; i < (kBackward ? 4 : 2); ++i) sidx[i] = static_cast<uint32_t>(w_flat[i] % g.period);
+    }
+  }
+  const int steps = static_cast<int>(R / BR);
+  const int last = steps - 1;
+  auto tile_r0 = [&](int t) { return static_cast<int64_t>(t < last ? t : last) * BR; };   // clamped: reloading the last tile is harmless
+  auto load_w = [&](auto set_, int t) {
     constexpr int set = decltype(set_)::value;
+    const int64_t r0 = tile_r0(t);
+    if constexpr (!kInt4) {
+      if (g.scale_mode == SM_VEC4) {
+        constexpr int rows = kBackward ? 4 : 2;
+        constexpr int quads = kBackward ? 2 : 4;
+#pragma unroll
+        for (int i = 0; i < rows; ++i) {
+#pragma unroll
+          for (int q = 0; q < quads; ++q) {
+            uint32_t idx = sidx[i] + 4 * q;
+            if (idx >= period32) idx -= period32;
+            wsc8[set][quads * i + q] = *reinterpret_cast<const floatx4_t *>(s32 + idx);
+          }
+          if (t < last) {
+            sidx[i] += g.scale_step;
+            if (sidx[i] >= period32) sidx[i] -= period32;
+          }
+        }
+      }
+    }
     if constexpr (!kBackward) {
       if constexpr (kInt4) {
         const int64_t f = w_flat[0] + r0;
@@ -256,11 +295,10 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
     }
   };
   // int8: fp32 value of 4 codes of dword p whose first code has flat index f
-  auto deq8 = [&](uint32_t p, int64_t f, float (&out)[4]) {
+  auto deq8 = [&](uint32_t p, const floatx4_t &s, int64_t f, float (&out)[4]) {
     float q[4];
     int8x4_to_f32(p, q);
     if (g.scale_mode == SM_VEC4) {
-      const floatx4_t s = *reinterpret_cast<const floatx4_t *>(s32 + (f % g.period));
 #pragma unroll
       for (int j = 0; j < 4; ++j) out[j] = q[j] * s[j];
     } else {
@@ -287,8 +325,8 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
         const int i = part >> 1;
         const int j = part & 1;
         float lo[4], hi[4];
-        deq8(wreg[set][4 * i + 2 * j], w_flat[i] + r0 + 8 * j, lo);
-        deq8(wreg[set][4 * i + 2 * j + 1], w_flat[i] + r0 + 8 * j + 4, hi);
+        deq8(wreg[set][4 * i + 2 * j], wsc8[set][4 * i + 2 * j], w_flat[i] + r0 + 8 * j, lo);
+        deq8(wreg[set][4 * i + 2 * j + 1], wsc8[set][4 * i + 2 * j + 1], w_flat[i] + r0 + 8 * j + 4, hi);
         u32x4_t v;
         v[0] = pack2<CT>(lo[0], lo[1]);
         v[1] = pack2<CT>(lo[2], lo[3]);
@@ -303,8 +341,8 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
       } else {
         const int64_t f = w_flat[i] + r0 * g.K;
         float lo[4], hi[4];
-        deq8(wreg[set][2 * i], f, lo);
-        deq8(wreg[set][2 * i + 1], f + 4, hi);
+        deq8(wreg[set][2 * i], wsc8[set][2 * i], f, lo);
+        deq8(wreg[set][2 * i + 1], wsc8[set][2 * i + 1], f + 4, hi);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           et[i][j] = lo[j];
@@ -325,6 +363,51 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
   };
 
   // ---- main loop ------------------------------------------------------------------------
+  // Wave specialisation: the four producer waves move tile s+1 from their registers into LDS
+  // buffer (s+1)&1 (dequantising W on the way) and fetch tile s+2 from global memory, while the
+  // four consumer waves run the MFMAs of tile s out of buffer s&1.  One producer and one consumer
+  // wave share each SIMD, so the VALU work of unpacking and the matrix pipe overlap without any
+  // instruction-level interleaving; all eight waves meet at one barrier per step.
+  typedef std::integral_constant<int, 0> I0;
+  typedef std::integral_constant<int, 1> I1;
+
+  if (producer) {
+    load_a(I0{}, 0);
+    load_w(I0{}, 0);
+#pragma unroll
+    for (int part = 0; part < 4; ++part) {
+      store_a(I0{}, smem, part);
+      store_w(I0{}, smem + kBBase, 0, part);
+    }
+    load_a(I1{}, tile_r0(1));
+    load_w(I1{}, 1);
+    load_a(I0{}, tile_r0(2));
+    load_w(I0{}, 2);
+    __syncthreads();
+    // step s: register set (s+1)&1 holds tile s+1 -> LDS buffer (s+1)&1, then that set <- tile s+3
+    // (set p always carries tiles of parity p; a load has two steps to arrive)
+    auto pstep = [&](auto buf_, int s) {
+      constexpr int buf = decltype(buf_)::value;
+      typedef std::integral_constant<int, 1 - buf> NxtSet;
+      const int64_t r_next = tile_r0(s + 1);
+#pragma unroll
+      for (int part = 0; part < 4; ++part) {
+        store_a(NxtSet{}, smem + (1 - buf) * kATileBytes, part);
+        store_w(NxtSet{}, smem + kBBase + (1 - buf) * kBTileBytes, r_next, part);
+      }
+      load_a(NxtSet{}, tile_r0(s + 3));
+      load_w(NxtSet{}, s + 3);
+      __syncthreads();
+    };
+    int s = 0;
+    for (; s + 2 <= steps; s += 2) {
+      pstep(I0{}, s);
+      pstep(I1{}, s + 1);
+    }
+    if (s < steps) pstep(I0{}, s);
+    return;
+  }
+
   floatx16_t acc[WR][2];
 #pragma unroll
   for (int i = 0; i < WR; ++i)
@@ -333,38 +416,15 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  const int steps = static_cast<int>(R / BR);
-  const int last = steps - 1;
-  typedef std::integral_constant<int, 0> I0;
-  typedef std::integral_constant<int, 1> I1;
-  auto tile_r0 = [&](int t) { return static_cast<int64_t>(t < last ? t : last) * BR; };   // clamped: reloading the last tile is harmless
-
-  load_a(I0{}, 0);
-  load_w(I0{}, 0);
-#pragma unroll
-  for (int part = 0; part < 4; ++part) {
-    store_a(I0{}, smem, part);
-    store_w(I0{}, smem + kATileBytes, 0, part);
-  }
-  load_a(I1{}, tile_r0(1));
-  load_w(I1{}, tile_r0(1));
-  __syncthreads();
-
   const int frow = lane & 31;    // row of the operand tile this lane supplies
   const int fh = lane >> 5;      // which half of the 16-wide k step
-  int a_frag_off[WR], b_frag_off[2];   // LDS byte offsets of this lane's operand rows (chunk 0, before the swizzle)
-  // One step s: MFMAs on LDS buffer `buf` (= s & 1); the tile held in the other register set goes
-  // to the other buffer; register set `buf` is refilled with tile s+2.
-  auto step = [&](auto buf_, int s) {
-    constexpr int buf = decltype(buf_)::value;
-    typedef decltype(buf_) CurSet;
-    typedef std::integral_constant<int, 1 - buf> NxtSet;
-    const unsigned char *abuf = smem + buf * kStageBytes;
-    const unsigned char *bbuf = abuf + kATileBytes;
-    unsigned char *nbuf = smem + (1 - buf) * kStageBytes;
-    const int64_t r_next = tile_r0(s + 1);
-    load_a(CurSet{}, tile_r0(s + 2));
-    load_w(CurSet{}, tile_r0(s + 2));
+
+  __syncthreads();               // tile 0 is in LDS
+  auto cstep = [&](auto abuf_, auto bbuf_, int s) {
+    constexpr int astage = decltype(abuf_)::value;
+    constexpr int bstage = decltype(bbuf_)::value;
+    const unsigned char *abuf = smem + astage * kATileBytes;
+    const unsigned char *bbuf = smem + kBBase + bstage * kBTileBytes;
     // operand fragments are double buffered in registers: the reads of k step ks+1 are issued
     // before the MFMAs of k step ks
     vec_t af[2][WR], bf[2][2];
@@ -377,7 +437,6 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
         bf[fb][j] = *reinterpret_cast<const vec_t *>(bbuf + swz(wc * 64 + j * 32 + frow, ks * 2 + fh));
     };
     read_frags(0, 0);
-    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < BR / 16; ++ks) {
       const int fsel = ks & 1;
@@ -386,30 +445,17 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
       for (int i = 0; i < WR; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = Mfma32<CT>::run(af[fsel][i], bf[fsel][j], acc[i][j]);
-      store_a(NxtSet{}, nbuf, ks);
-      store_w(NxtSet{}, nbuf + kATileBytes, r_next, ks);
-      // Order inside the k step: next fragments' reads first, then every MFMA followed by a few
-      // VALU instructions of the dequantisation (one wave has to keep the matrix pipe and the VALU
-      // busy at the same time), LDS writes last.
-      if (ks + 1 < BR / 16) __builtin_amdgcn_sched_group_barrier(0x100, WR + 2, 0);
-#pragma unroll
-      for (int t = 0; t < WR * 2; ++t) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, kBackward ? 8 : 6, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x200, 16, 0);
-      __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
   };
-  (void)a_frag_off;
-  (void)b_frag_off;
-  int s = 0;
-  for (; s + 2 <= steps; s += 2) {
-    step(I0{}, s);
-    step(I1{}, s + 1);
+  {
+    int s = 0;
+    for (; s + 2 <= steps; s += 2) {
+      cstep(I0{}, I0{}, s);
+      cstep(I1{}, I1{}, s + 1);
+    }
+    if (s < steps) cstep(I0{}, I0{}, s);
   }
-  if (s < steps) step(I0{}, s);
 
   // ---- epilogue: acc[i][j][r] = D[row][col], row = 8*(r/4) + 4*(lane/32) + r%4, col = lane%32
 #pragma unroll
@@ -454,16 +500,25 @@ int launch_one(const TileArgs &t, int64_t row_tiles, hipStream_t s)
   return launch_status();
 }
 
-// 128-row tiles everywhere: measured on MI355X, two or three resident workgroups per CU (64 KiB of
-// LDS and about 180 registers each) overlap one workgroup's dequantisation with another's MFMAs and
-// reach 1.4-1.9 PFLOP/s, while 256-row tiles (one workgroup per CU) stay near 0.75 PFLOP/s even
-// though they halve the dequantisation work per flop.
+// Tile height.  LDS bandwidth (128 B/clk per CU) is what bounds this kernel: a consumer wave reads
+// one 16-byte fragment per lane for every 32x32x16 MFMA it feeds, and with 64x64 wave tiles that is
+// one fragment read per MFMA.  256-row workgroup tiles (128x64 per consumer wave) need 0.75 reads
+// per MFMA and half the weight staging per flop, so they are used whenever there are enough of
+// them to fill the chip; expert segments (a few hundred rows each) keep 128-row tiles.
 template <typename CT, typename XT, bool kInt4, bool kBackward>
 int launch_tile(const TileArgs &t, bool grouped, hipStream_t s)
 {
-  const int64_t row_tiles = (t.M + 127) / 128 + (grouped ? t.num_experts : 0);   // every expert can add one partial tile
+  const int64_t C = kBackward ? t.K : t.N;
+  const int64_t col_tiles = (C + BC - 1) / BC;
+  if (grouped) {
+    const int64_t row_tiles = (t.M + 127) / 128 + t.num_experts;   // every expert can add one partial tile
+    if (row_tiles > 65535) return CAIFX_ERR_UNSUPPORTED;
+    return launch_one<CT, XT, kInt4, kBackward, true, 128>(t, row_tiles, s);
+  }
+  const int64_t tall = (t.M + 255) / 256;
+  if (tall * col_tiles >= 200 && tall <= 65535) return launch_one<CT, XT, kInt4, kBackward, false, 256>(t, tall, s);
+  const int64_t row_tiles = (t.M + 127) / 128;
   if (row_tiles > 65535) return CAIFX_ERR_UNSUPPORTED;
-  if (grouped) return launch_one<CT, XT, kInt4, kBackward, true, 128>(t, row_tiles, s);
   return launch_one<CT, XT, kInt4, kBackward, false, 128>(t, row_tiles, s);
 }
 
@@ -509,8 +564,10 @@ int run(const GemmArgs &a, bool backward, hipStream_t s)
     t.period = a.w.scale_period;
     if (!has_scales || t.period == 1) {
       t.scale_mode = SM_SCALAR;
-    } else if (t.period % 4 == 0 && (grouped || aligned_to(a.w.scales, 16))) {
+    } else if (t.period % 4 == 0 && t.period < (int64_t{1} << 31) && (grouped || aligned_to(a.w.scales, 16))) {
       t.scale_mode = SM_VEC4;     // flat index of every fetched quad is a multiple of 4 (K % 32 == 0)
+      // one step moves the flat index by 64 (forward: along k) or by 64 rows of K codes (backward)
+      t.scale_step = static_cast<uint32_t>((backward ? (static_cast<int64_t>(BR) * t.K) % t.period : BR % t.period));
     } else {
       t.scale_mode = SM_ANY;
     }
