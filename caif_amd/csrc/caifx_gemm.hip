@@ -110,6 +110,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
 
   // ---- which tile -----------------------------------------------------------------------
   int64_t row_lo, row_hi;        // rows of A / D this workgroup may touch: [row_lo, row_hi)
+  int64_t col_tile = blockIdx.x;
   const uint8_t *wq = static_cast<const uint8_t *>(g.wq);
   const void *scales = g.scales;
   if constexpr (kGrouped) {
@@ -134,10 +135,26 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
     wq = static_cast<const uint8_t *>(g.wq_ptrs[e]);
     scales = g.scales_ptrs ? g.scales_ptrs[e] : nullptr;
   } else {
-    row_lo = static_cast<int64_t>(blockIdx.y) * BM;
+    // Workgroups are handed to the 8 XCDs in turn (linear id mod 8), and each XCD has its own L2.
+    // The tiles are therefore numbered so that one XCD walks one contiguous eighth of the list, and
+    // the list runs through bands of 512 rows column by column: the 32 tiles an XCD works on at any
+    // time form a 512-row x 16-tile patch, which touches far fewer distinct rows of A than a
+    // full-height stripe of the same area.  The grid is padded to a multiple of 8.
+    constexpr int kBandTiles = 512 / BM;
+    const int64_t col_tiles = (C + BC - 1) / BC;
+    const int64_t row_tiles = (g.M + BM - 1) / BM;
+    const int64_t per_xcd = gridDim.x >> 3;
+    const int64_t pos = static_cast<int64_t>(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (pos >= row_tiles * col_tiles) return;
+    const int64_t band = pos / (kBandTiles * col_tiles);
+    const int64_t within = pos - band * kBandTiles * col_tiles;
+    const int64_t left = row_tiles - band * kBandTiles;
+    const int64_t band_rows = left < kBandTiles ? left : kBandTiles;
+    col_tile = within / band_rows;
+    row_lo = (band * kBandTiles + within % band_rows) * BM;
     row_hi = g.M;
   }
-  const int64_t col0 = static_cast<int64_t>(blockIdx.x) * BC;
+  const int64_t col0 = col_tile * BC;
   const XT *ag = static_cast<const XT *>(g.a);
 
   // ---- global -> register staging ---------------------------------------------------------
@@ -495,7 +512,13 @@ int launch_one(const TileArgs &t, int64_t row_tiles, hipStream_t s)
       raised = true;
     }
   }
-  dim3 grid(static_cast<unsigned>((C + BC - 1) / BC), static_cast<unsigned>(row_tiles));
+  const int64_t col_tiles = (C + BC - 1) / BC;
+  dim3 grid(static_cast<unsigned>(col_tiles), static_cast<unsigned>(row_tiles));
+  if (!kGrouped) {
+    const int64_t padded = (row_tiles * col_tiles + 7) / 8 * 8;      // linear grid, see the tile numbering in the kernel
+    if (padded > 0x7fffffff) return CAIFX_ERR_UNSUPPORTED;
+    grid = dim3(static_cast<unsigned>(padded), 1);
+  }
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds, s, t);
   return launch_status();
 }
