@@ -101,11 +101,19 @@ int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K, const void *x, int x_
   const GemmArgs a = make_args(M, N, K, x, x_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, y,
                                y_dtype, workspace, workspace_bytes);
   hipStream_t s = as_stream(stream);
-  if (M <= 4) {
+  // one or two rows: stream each weight row linearly and reduce per row; from three rows on the
+  // matrix-core tiling (cost independent of M) is faster; both fall through when a shape does not fit
+  if (M <= 2) {
     st = rowlin_forward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return st;
   }
   if (M <= 16) {
+    st = mblock_forward(a, s);
+    if (st != CAIFX_ERR_UNSUPPORTED) return st;
+    if (M <= 4) {
+      st = rowlin_forward(a, s);
+      if (st != CAIFX_ERR_UNSUPPORTED) return st;
+    }
     st = skinny_forward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return st;
   }

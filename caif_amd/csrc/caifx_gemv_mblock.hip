@@ -1,0 +1,397 @@
+// Decode path for a handful of activation rows (2 <= M <= 16): Y[M,N] = X[M,K] * W[N,K]^T with W
+// stored int8 or packed int4, memory bound on the weight stream.
+//
+// The matrix cores do the dot products with the activation rows as the 16 rows of the A operand
+// of v_mfma_f32_16x16x32 (rows past M are zero) and 16 weight rows as the columns of B, so the
+// cost per weight byte does not depend on M.  A workgroup is 16 waves; wave w owns the k range
+// [w*GPW*128, (w+1)*GPW*128) for every weight row the workgroup visits and keeps the matching
+// slice of X in registers, already laid out as A operands, for the whole kernel.  Per block of 16
+// weight rows a lane (j = lane%16, q = lane/16) loads 16 bytes of row j:
+//   int4: 32 codes at k = group*128 + q*32; dword t of the load feeds MFMA t, its nibbles unpack
+//         pairwise (order 0,4,1,5,2,6,3,7, X is stored in the same order) to the compute dtype as
+//         OFFSET + (code + 8) with one AND/XOR each; the fp32 sum over a 128-k group is corrected by
+//         OFFSET' * sum(x) and multiplied by the group's scale ("post-scaling": the weight is never
+//         rounded to the compute dtype, so results differ from the dequantise-then-cast reference
+//         by that rounding, a few 1e-3 of the largest output);
+//   int8: 16 codes at k = group*128 + half*64 + q*16, each multiplied by its scale in fp32 and
+//         rounded once to the compute dtype, exactly as the reference forms its weight.  A scale
+//         vector of period P is addressed by the flat index n*K + k modulo P; rows n with equal
+//         n mod V, V = P / gcd(K mod P, P), see the same scales along k, so a workgroup only visits rows
+//         of one residue class and keeps that class's K scales in LDS.
+// After the last group every wave holds a partial 16x16 tile; the 16 partials are added through LDS
+// in a fixed order (results do not depend on scheduling) and written as Y[token][row].
+#include "caifx_internal.hpp"
+
+namespace caifx {
+namespace {
+
+template <typename CT> struct Mfma16;
+template <> struct Mfma16<bf16_t> {
+  typedef bf16x8_t vec_t;
+  static constexpr uint32_t kMagic = 0x43084308u;      // bf16 128 + (code ^ 8) in both halves
+  static constexpr float kOffset = 136.0f;             // 128 + 8
+  static __device__ __forceinline__ floatx4_t run(vec_t a, vec_t b, floatx4_t c)
+  {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma16<f16_t> {
+  typedef f16x8_t vec_t;
+  static constexpr uint32_t kMagic = 0x64086408u;      // fp16 1024 + (code ^ 8)
+  static constexpr float kOffset = 1032.0f;
+  static __device__ __forceinline__ floatx4_t run(vec_t a, vec_t b, floatx4_t c)
+  {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+constexpr int kMbWaves = 16;
+constexpr int kMbThreads = kMbWaves * 64;
+constexpr int kPartialFloats = kMbWaves * 4 * 64;     // one buffer of per-wave partial tiles
+
+struct MbArgs {
+  const uint8_t *wq;
+  const void *scales;
+  const void *x;
+  void *y;
+  int M;
+  int y_dtype;
+  int64_t N, K;
+  int groups;            // K / 128
+  int group_shift;       // int4: log2(group_size)
+  int period;            // int8: length of the scale vector, 0 = one scale (or none)
+  int V;                 // residue classes the rows are split into (1 unless period > 0)
+  int blocks_per_class;  // gridDim.x = blocks_per_class * V
+  int scale_step;        // int8 scale vector: 1024 mod period (staging stride of the workgroup)
+};
+
+// 8 consecutive activations as compute-dtype values
+template <typename CT, typename XT>
+__device__ __forceinline__ typename Mfma16<CT>::vec_t load_x8(const XT *p)
+{
+  typedef typename Mfma16<CT>::vec_t vec_t;
+  if constexpr (dtype_code<XT>::value == dtype_code<CT>::value) {
+    return *reinterpret_cast<const vec_t *>(p);
+  } else if constexpr (sizeof(XT) == 4) {
+    const floatx4_t a = *reinterpret_cast<const floatx4_t *>(p);
+    const floatx4_t b = *reinterpret_cast<const floatx4_t *>(p + 4);
+    vec_t v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[i] = from_f32<CT>(a[i]);
+      v[4 + i] = from_f32<CT>(b[i]);
+    }
+    return v;
+  } else {
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(p);
+    const XT *h = reinterpret_cast<const XT *>(&raw);
+    vec_t v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = from_f32<CT>(to_f32<XT>(h[i]));
+    return v;
+  }
+}
+
+__device__ __forceinline__ void store_out(void *y, int y_dtype, int64_t o, float v)
+{
+  if (y_dtype == CAIFX_F32) static_cast<float *>(y)[o] = v;
+  else if (y_dtype == CAIFX_BF16) static_cast<bf16_t *>(y)[o] = from_f32<bf16_t>(v);
+  else static_cast<f16_t *>(y)[o] = from_f32<f16_t>(v);
+}
+
+// GPW: 128-k groups per wave (K <= 16 * GPW * 128); 1 and 2 fit the 128 registers of a 1024-thread workgroup
+template <typename CT, typename XT, bool kInt4, int GPW>
+__global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
+{
+  typedef typename Mfma16<CT>::vec_t vec_t;
+  constexpr int LPG = kInt4 ? 1 : 2;           // 16-byte loads per lane per 128-k group
+  constexpr int LPR = GPW * LPG;               // ... per block of 16 weight rows
+  constexpr int D = LPR >= 4 ? 1 : 4 / LPR;    // row blocks in flight (4 loads per lane)
+  constexpr int RBB = kInt4 ? 4 : 2;           // row blocks between two reductions (a multiple of D)
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float *partial = reinterpret_cast<float *>(smem);      // [RBB][16 waves][4][64]
+  float *svec = partial + RBB * kPartialFloats;          // int8 with a scale vector: [K]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int j = lane & 15;        // weight row within the block (B column) / activation row (A row)
+  const int q = lane >> 4;        // quarter of the 32-wide k step
+  const int cls = blockIdx.x / a.blocks_per_class;
+  const int bc = blockIdx.x - cls * a.blocks_per_class;
+  const int64_t rows_class = (a.N - cls + a.V - 1) / a.V;          // rows n = cls + V*i, i < rows_class
+  // every workgroup of a class takes the same number of consecutive rows (the last block of 16 may
+  // be partly masked): equal bytes per compute unit matter more than full MFMA tiles
+  const int64_t per_block = (rows_class + a.blocks_per_class - 1) / a.blocks_per_class;
+  const int64_t i_lo = bc * per_block;
+  const int64_t i_hi = i_lo + per_block < rows_class ? i_lo + per_block : rows_class;
+  const int nrb = i_hi > i_lo ? static_cast<int>((i_hi - i_lo + 15) / 16) : 0;
+  const int g0 = wave * GPW;
+  const f16_t *s16 = static_cast<const f16_t *>(a.scales);
+  const float *s32 = static_cast<const float *>(a.scales);
+
+  u32x4_t w[D][LPR];
+  f16_t sc[D][GPW];
+  auto issue = [&](int d, int rb) {
+    const int64_t i = i_lo + static_cast<int64_t>(rb) * 16 + j;
+    if (i < i_hi) {                    // masked lanes fetch nothing; their columns of the tile are never stored
+      const int64_t f0 = (cls + a.V * i) * a.K;
+#pragma unroll
+      for (int g = 0; g < GPW; ++g) {
+        const int gg = g0 + g;
+        if (gg < a.groups) {
+          const int64_t f = f0 + gg * 128;
+          if constexpr (kInt4) {
+            w[d][g] = *reinterpret_cast<const u32x4_t *>(a.wq + (f >> 1) + q * 16);
+            sc[d][g] = s16[f >> a.group_shift];
+          } else {
+            w[d][2 * g] = *reinterpret_cast<const u32x4_t *>(a.wq + f + q * 16);
+            w[d][2 * g + 1] = *reinterpret_cast<const u32x4_t *>(a.wq + f + 64 + q * 16);
+          }
+        }
+      }
+    }
+  };
+  // Order of the requests: this wave's slice of X first (it comes from L2 and is needed first),
+  // then the first weight blocks; loads return in order, so X can be turned into A operands while
+  // the weights are still on their way from HBM.
+  vec_t xa[GPW][4];
+  {
+    const XT *xg = static_cast<const XT *>(a.x) + static_cast<int64_t>(j < a.M ? j : 0) * a.K;
+#pragma unroll
+    for (int g = 0; g < GPW; ++g) {
+      const int gg = g0 + g;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        vec_t v;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = from_f32<CT>(0.0f);
+        if (gg < a.groups && j < a.M) {
+          const int k = kInt4 ? gg * 128 + q * 32 + 8 * t : gg * 128 + (t >> 1) * 64 + q * 16 + 8 * (t & 1);
+          v = load_x8<CT, XT>(xg + k);
+        }
+        xa[g][t] = v;
+      }
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < nrb) issue(d, d);
+
+  // int8 scale vector of this residue class: svec[k] = scales[(cls*K + k) mod period]
+  float s_one = 1.0f;
+  if constexpr (!kInt4) {
+    if (a.period > 0) {
+      int idx = static_cast<int>((static_cast<int64_t>(cls) * a.K + threadIdx.x) % a.period);
+      for (int64_t k = threadIdx.x; k < a.K; k += kMbThreads) {
+        svec[k] = s32[idx];
+        idx += a.scale_step;
+        if (idx >= a.period) idx -= a.period;
+      }
+    } else if (a.scales) {
+      s_one = s32[0];
+    }
+  }
+
+  // int4: the nibbles unpack in the order 0,4,1,5,2,6,3,7, so X is stored that way; and
+  // cor = OFFSET * (sum of x over each group) for the four activation rows this lane holds results of
+  float cor[GPW][4];
+  if constexpr (kInt4) {
+    vec_t ones;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ones[i] = from_f32<CT>(1.0f);
+#pragma unroll
+    for (int g = 0; g < GPW; ++g) {
+      // the group sums come out of the matrix core in the layout of the results: X times a matrix of ones
+      floatx4_t xsum = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const vec_t v = xa[g][t];
+        xsum = Mfma16<CT>::run(v, ones, xsum);
+        vec_t p;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          p[2 * i] = v[i];
+          p[2 * i + 1] = v[i + 4];
+        }
+        xa[g][t] = p;
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) cor[g][r] = Mfma16<CT>::kOffset * xsum[r];
+    }
+  }
+  if constexpr (!kInt4) __syncthreads();       // svec is complete
+
+  // The waves run freely through RBB blocks of 16 rows (no barrier in between, so one wave's
+  // arithmetic overlaps another's wait for HBM), then the 16 partial tiles of each block are added
+  // through LDS in a fixed order.
+  for (int base = 0; base < nrb; base += RBB) {
+    floatx4_t tot[RBB];
+#pragma unroll
+    for (int u = 0; u < RBB; ++u) {
+      const int d = u % D;
+      const int rb = base + u;
+      tot[u] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      if (rb < nrb) {          // same for every thread of the workgroup
+        u32x4_t wr[LPR];
+        float sr[GPW];
+#pragma unroll
+        for (int i = 0; i < LPR; ++i) wr[i] = w[d][i];
+        if constexpr (kInt4) {
+#pragma unroll
+          for (int g = 0; g < GPW; ++g) sr[g] = to_f32(sc[d][g]);
+        }
+        if (rb + D < nrb) issue(d, rb + D);
+#pragma unroll
+        for (int g = 0; g < GPW; ++g) {
+          const int gg = g0 + g;
+          if (gg < a.groups) {
+            if constexpr (kInt4) {
+              floatx4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                const uint32_t p = wr[g][t];
+                u32x4_t c4;
+                c4[0] = (p & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
+                c4[1] = ((p >> 4) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
+                c4[2] = ((p >> 8) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
+                c4[3] = ((p >> 12) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
+                acc = Mfma16<CT>::run(xa[g][t], *reinterpret_cast<const vec_t *>(&c4), acc);
+              }
+#pragma unroll
+              for (int r = 0; r < 4; ++r) tot[u][r] = __builtin_fmaf(sr[g], acc[r] - cor[g][r], tot[u][r]);
+            } else {
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                float lo[4], hi[4];
+                int8x4_to_f32(wr[2 * g + (t >> 1)][2 * (t & 1)], lo);
+                int8x4_to_f32(wr[2 * g + (t >> 1)][2 * (t & 1) + 1], hi);
+                floatx4_t s0 = {s_one, s_one, s_one, s_one};
+                floatx4_t s1 = s0;
+                if (a.period > 0) {
+                  const float *sp = svec + gg * 128 + (t >> 1) * 64 + q * 16 + 8 * (t & 1);
+                  s0 = *reinterpret_cast<const floatx4_t *>(sp);
+                  s1 = *reinterpret_cast<const floatx4_t *>(sp + 4);
+                }
+                vec_t bv;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                  bv[i] = from_f32<CT>(lo[i] * s0[i]);
+                  bv[4 + i] = from_f32<CT>(hi[i] * s1[i]);
+                }
+                tot[u] = Mfma16<CT>::run(xa[g][t], bv, tot[u]);
+              }
+            }
+          }
+        }
+      }
+    }
+
+    // tot[u][r] = this wave's share of Y[activation row 4q+r][weight row j of block base+u]
+#pragma unroll
+    for (int u = 0; u < RBB; ++u)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) partial[((u * kMbWaves + wave) * 4 + r) * 64 + lane] = tot[u][r];
+    __syncthreads();
+    if (threadIdx.x < RBB * 256) {
+      const int u = threadIdx.x >> 8;
+      const int r = (threadIdx.x >> 6) & 3;
+      const int l = threadIdx.x & 63;
+      float v = 0.0f;
+#pragma unroll
+      for (int wv = 0; wv < kMbWaves; ++wv) v += partial[((u * kMbWaves + wv) * 4 + r) * 64 + l];
+      const int m = 4 * (l >> 4) + r;
+      const int64_t i = i_lo + static_cast<int64_t>(base + u) * 16 + (l & 15);
+      if (m < a.M && i < i_hi) store_out(a.y, a.y_dtype, static_cast<int64_t>(m) * a.N + cls + a.V * i, v);
+    }
+    if (base + RBB < nrb) __syncthreads();      // the next round overwrites the partial tiles
+  }
+}
+
+int64_t gcd64(int64_t x, int64_t y)
+{
+  while (y) {
+    const int64_t t = x % y;
+    x = y;
+    y = t;
+  }
+  return x;
+}
+
+template <typename CT, typename XT, bool kInt4>
+int launch_gpw(const MbArgs &m, size_t lds, hipStream_t s)
+{
+  const unsigned grid = static_cast<unsigned>(m.blocks_per_class * m.V);
+  const int gpw = (m.groups + kMbWaves - 1) / kMbWaves;
+  if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 1>), dim3(grid), dim3(kMbThreads), lds, s, m);
+  else if (gpw <= 2) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 2>), dim3(grid), dim3(kMbThreads), lds, s, m);
+  else return CAIFX_ERR_UNSUPPORTED;
+  return launch_status();
+}
+
+template <typename CT>
+int launch_xt(const MbArgs &m, int x_dtype, bool int4, size_t lds, hipStream_t s)
+{
+  if (x_dtype == CAIFX_F32) return int4 ? launch_gpw<CT, float, true>(m, lds, s) : launch_gpw<CT, float, false>(m, lds, s);
+  if (x_dtype == CAIFX_F16) return int4 ? launch_gpw<CT, f16_t, true>(m, lds, s) : launch_gpw<CT, f16_t, false>(m, lds, s);
+  return int4 ? launch_gpw<CT, bf16_t, true>(m, lds, s) : launch_gpw<CT, bf16_t, false>(m, lds, s);
+}
+
+int compute_units()
+{
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = 256;
+  }
+  return cus;
+}
+
+}  // namespace
+
+int mblock_forward(const GemmArgs &g, hipStream_t s)
+{
+  if (g.offsets || g.M < 1 || g.M > 16 || g.compute_dtype == CAIFX_F32) return CAIFX_ERR_UNSUPPORTED;
+  if (g.N < 16 || g.N > (int64_t{1} << 30) || g.K % 128 != 0 || g.K > kMbWaves * 2 * 128) return CAIFX_ERR_UNSUPPORTED;
+  if (!aligned_to(g.w.q, 16) || !aligned_to(g.x, 16)) return CAIFX_ERR_UNSUPPORTED;
+  const bool int4 = g.w.kind == CAIFX_W_INT4_GROUP;
+
+  MbArgs m{};
+  m.wq = static_cast<const uint8_t *>(g.w.q);
+  m.scales = g.w.scales;
+  m.x = g.x;
+  m.y = g.y;
+  m.M = static_cast<int>(g.M);
+  m.y_dtype = g.y_dtype;
+  m.N = g.N;
+  m.K = g.K;
+  m.groups = static_cast<int>(g.K / 128);
+  m.V = 1;
+  size_t lds = (int4 ? 4 : 2) * kPartialFloats * sizeof(float);      // RBB buffers of partial tiles
+  if (int4) {
+    const int gs = g.w.group_size;
+    if (!g.w.scales || gs < 128 || (gs & (gs - 1)) != 0) return CAIFX_ERR_UNSUPPORTED;
+    m.group_shift = __builtin_ctz(static_cast<unsigned>(gs));
+  } else if (g.w.scales && g.w.scale_period > 1) {
+    const int64_t P = g.w.scale_period;
+    if (P > (int64_t{1} << 30) || !aligned_to(g.w.scales, 4)) return CAIFX_ERR_UNSUPPORTED;
+    const int64_t V = P / gcd64(g.K % P == 0 ? P : g.K % P, P);
+    if (V * 64 > g.N) return CAIFX_ERR_UNSUPPORTED;      // too few rows per residue class
+    m.period = static_cast<int>(P);
+    m.scale_step = static_cast<int>(kMbThreads % P);
+    m.V = static_cast<int>(V);
+    lds += static_cast<size_t>(g.K) * sizeof(float);
+  }
+  int target = compute_units();
+  const int64_t nrb_class = ((g.N + m.V - 1) / m.V + 15) / 16;
+  int64_t bpc = target / m.V;
+  if (bpc < 1) bpc = 1;
+  if (bpc > nrb_class) bpc = nrb_class;        // at least 16 rows per workgroup
+  m.blocks_per_class = static_cast<int>(bpc);
+  if (g.compute_dtype == CAIFX_BF16) return launch_xt<bf16_t>(m, g.x_dtype, int4, lds, s);
+  return launch_xt<f16_t>(m, g.x_dtype, int4, lds, s);
+}
+
+}  // namespace caifx

@@ -39,6 +39,9 @@ int generic_backward(const GemmArgs &a, hipStream_t s);
 int skinny_forward(const GemmArgs &a, hipStream_t s);
 // M <= 4 decode path that streams each weight row linearly (the fastest access pattern).
 int rowlin_forward(const GemmArgs &a, hipStream_t s);
+// M <= 16 decode path on the matrix cores: activation rows are the A operand, so the cost per
+// weight byte does not grow with M.
+int mblock_forward(const GemmArgs &a, hipStream_t s);
 
 // Large-M MFMA path (compute bound), forward and input gradient, plain and grouped.
 int mfma_forward(const GemmArgs &a, hipStream_t s);

@@ -66,6 +66,17 @@ def test_ragged_and_wave_count_variants(orc, N, K, M):
     _check(orc, rng, M, N, K, "int8pc", 2, 2)
 
 
+@pytest.mark.parametrize("N,K,M", [(1536, 1024, 6), (14336, 4096, 4), (200, 4096, 3), (2050, 640, 11)])
+def test_residue_classes_and_masked_row_blocks(orc, N, K, M):
+    # 3 <= M <= 16 runs on the matrix cores in blocks of 16 weight rows: N = 200 and 2050 leave a
+    # partly masked last block; int8 per-channel scales (period N) split the rows into
+    # N / gcd(K mod N, N) residue classes: 3 for (1536, 1024), 7 for the full decode shape
+    rng = np.random.default_rng(N * 7 + K + M)
+    _check(orc, rng, M, N, K, "int4", 2, 2)
+    _check(orc, rng, M, N, K, "int8pc", 2, 2)
+    _check(orc, rng, M, N, K, "int8pt", 1, 0)
+
+
 @pytest.mark.parametrize("group", [32, 64, 256, 512])
 def test_int4_group_sizes(orc, group):
     _check(orc, np.random.default_rng(group), 2, 128, 1024, "int4", 2, 2, group=group)
