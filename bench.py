@@ -12,8 +12,8 @@ The launches of the timed region are captured once into a HIP graph and replayed
 not the Python launch path, sets the pace; per-kernel durations for the roofline object come
 from HIP events around single-kernel graphs on the same stream.
 
-Also reported in `extra`: M in {4,16} decode rates, the cache-resident M=1 rate, and the
-compute-bound rows (configs[2..4]) in TFLOP/s.
+Also reported in `extra`: M in {4,16} decode rates, the cache-resident M=1 rate, the
+compute-bound rows (configs[2..3]) in TFLOP/s and the MoE frozen-expert layer (configs[4]) in tokens/s.
 """
 import argparse
 import json
@@ -240,7 +240,69 @@ def compute_bound_rows(torch, T, dev, gen, capture, time_graph):
             rows[key].update({"dx_us": round(ms_b * 1e3, 2), "dx_TFLOPs": round(flops / (ms_b * 1e-3) / 1e12, 1),
                               "fwd_dx_frac_of_mfma_peak":
                                   round(2 * flops / ((ms_f + ms_b) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
-    return {"prefill_gemm": rows}
+    return {"prefill_gemm": rows, "moe_frozen_experts": moe_rows(torch, T, dev, gen)}
+
+
+def moe_rows(torch, T, dev, gen):
+    """configs[4]: 64 frozen SwiGLU experts (int8 per-channel, gate/up 2048->1408, down 1408->2048), 4096
+    bf16 tokens, top-6 routing with uniform random expert ids: forward + backward dX as grouped
+    dequant-GEMMs over the token-sorted buffer.  Eager launches timed with HIP events."""
+    E, D, H, tokens, top_k = 64, 2048, 1408, 4096, 6
+
+    def bank(n, k):
+        ws = []
+        for _ in range(E):
+            w = torch.empty(k, n, device=dev).normal_(0, 0.02, generator=gen)     # the reference's [in,out] labelling
+            q, s = T.quantize_int8(w, per_channel=True)
+            ws.append(T.FrozenWeight(q.reshape(-1), T.W_INT8, s, n, k, n))
+        return T.GroupedFrozenWeights(ws)
+
+    gate, up, down = bank(H, D), bank(H, D), bank(D, H)
+    ids = torch.randint(0, E, (tokens * top_k,), device=dev, generator=gen)
+    counts = torch.bincount(ids, minlength=E)
+    offsets = torch.zeros(E + 1, dtype=torch.int32, device=dev)
+    offsets[1:] = torch.cumsum(counts, 0).to(torch.int32)
+    rows = tokens * top_k
+    x = torch.empty(rows, D, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16)
+    gout = torch.empty(rows, D, device=dev).normal_(0, 1e-2, generator=gen).to(torch.bfloat16)
+    bf = lambda r, c: torch.empty(r, c, dtype=torch.bfloat16, device=dev)
+    up_o, gate_o, out, gh, gi_up, gi_gate = bf(rows, H), bf(rows, H), bf(rows, D), bf(rows, H), bf(rows, D), bf(rows, D)
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    state = {}
+
+    def fwd():
+        T.qlinear_grouped_forward(x, offsets, up, T.BF16, T.BF16, out=up_o, workspace=ws)
+        T.qlinear_grouped_forward(x, offsets, gate, T.BF16, T.BF16, out=gate_o, workspace=ws)
+        state["hidden"] = T.silu_multiply(gate_o, up_o)
+        T.qlinear_grouped_forward(state["hidden"], offsets, down, T.BF16, T.BF16, out=out, workspace=ws)
+
+    def bwd():
+        T.qlinear_grouped_backward_input(gout, offsets, down, T.BF16, T.BF16, out=gh, workspace=ws)
+        grad_up = T.multiply(gh, T.silu(gate_o))
+        grad_gate = T.silu_backward(gate_o, T.multiply(gh, up_o))
+        T.qlinear_grouped_backward_input(grad_up, offsets, up, T.BF16, T.BF16, out=gi_up, workspace=ws)
+        T.qlinear_grouped_backward_input(grad_gate, offsets, gate, T.BF16, T.BF16, out=gi_gate, workspace=ws)
+        state["dx"] = T.add(gi_up, gi_gate)
+
+    def timed(fn, iters=10):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    ms_f, ms_b = timed(fwd), timed(bwd)
+    gemm_flops = 3 * 2.0 * rows * D * H
+    return {"experts": E, "tokens": tokens, "top_k": top_k, "packed_rows": rows,
+            "rows_per_expert_min_max": [int(counts.min()), int(counts.max())],
+            "fwd_ms": round(ms_f, 4), "bwd_ms": round(ms_b, 4),
+            "tokens_per_s_fwd_bwd": round(tokens / ((ms_f + ms_b) * 1e-3), 1),
+            "grouped_gemm_TFLOPs_fwd": round(gemm_flops / (ms_f * 1e-3) / 1e12, 1),
+            "grouped_gemm_TFLOPs_bwd": round(gemm_flops / (ms_b * 1e-3) / 1e12, 1)}
 
 
 def cpu_baseline(np, q8, s8, p4, s4_bits, x_values):

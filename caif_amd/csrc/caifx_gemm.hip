@@ -88,13 +88,17 @@ __device__ __forceinline__ float int8_scale_at(const float *scales, int mode, in
 }
 
 // BM: rows of D per workgroup (128 or 256); a wave owns (BM/2) x 64 of D.
-template <typename CT, typename XT, bool kInt4, bool kBackward, bool kGrouped, int BM>
-__global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
+// kSLds (int8 with a periodic scale vector that fits): the scale vector sits in LDS behind the
+// tile buffers and is read when a weight piece is dequantised, instead of travelling through
+// registers with the codes.
+template <typename CT, typename XT, bool kInt4, bool kSLds, bool kBackward, bool kGrouped, int BM>
+__global__ __launch_bounds__(kThreads, (BM == 128 && (kInt4 || kSLds)) ? 4 : 2) void qgemm_kernel(TileArgs g)
 {
   typedef typename Mfma32<CT>::vec_t vec_t;
   constexpr int kATileBytes = BM * BR * 2;
   constexpr int kAStages = 2;
   constexpr int kBBase = kAStages * kATileBytes;             // LDS: A ring, then two B buffers
+  constexpr int kSBase = kBBase + 2 * kBTileBytes;           // ... then the int8 scale vector (kSLds)
   constexpr int WR = BM / 64;                                // 32-row MFMA tiles per wave along M
   constexpr int kAChunks = BM / 32;                          // 16-byte LDS chunks of A per thread per step
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];          // 2 x kStageBytes
@@ -114,20 +118,38 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
   const uint8_t *wq = static_cast<const uint8_t *>(g.wq);
   const void *scales = g.scales;
   if constexpr (kGrouped) {
-    // blockIdx.y counts row tiles over all experts; find the expert by walking the offsets
+    // blockIdx.y counts row tiles over all experts.  Every wave finds the expert on its own: lane l
+    // takes expert base+l, an inclusive scan over the lanes gives the running tile count, and the
+    // first lane whose count exceeds blockIdx.y owns the tile.
     int t = blockIdx.y;
     int e = 0;
     int64_t lo = 0, hi = 0;
     bool found = false;
-    for (; e < g.num_experts; ++e) {
-      lo = g.offsets[e];
-      hi = g.offsets[e + 1];
-      const int tiles = static_cast<int>((hi - lo + BM - 1) / BM);
-      if (t < tiles) {
-        found = true;
-        break;
+    for (int base = 0; base < g.num_experts && !found; base += 64) {
+      const int my = base + lane;
+      int my_lo = 0, my_hi = 0;
+      if (my < g.num_experts) {
+        my_lo = g.offsets[my];
+        my_hi = g.offsets[my + 1];
       }
-      t -= tiles;
+      const int tiles = (my_hi - my_lo + BM - 1) / BM;
+      int incl = tiles;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+      }
+      const unsigned long long owners = __ballot(incl > t);
+      if (owners != 0) {
+        const int src = __builtin_ctzll(owners);
+        e = base + src;
+        t -= __shfl(incl - tiles, src, 64);
+        lo = __shfl(my_lo, src, 64);
+        hi = __shfl(my_hi, src, 64);
+        found = true;
+      } else {
+        t -= __shfl(incl, 63, 64);
+      }
     }
     if (!found) return;
     row_lo = lo + static_cast<int64_t>(t) * BM;
@@ -156,6 +178,13 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
   }
   const int64_t col0 = col_tile * BC;
   const XT *ag = static_cast<const XT *>(g.a);
+  float *slds = reinterpret_cast<float *>(smem + kSBase);
+  if constexpr (kSLds) {
+    const floatx4_t *src = static_cast<const floatx4_t *>(scales);
+    for (int i = threadIdx.x; i < static_cast<int>(g.period >> 2); i += kThreads)
+      reinterpret_cast<floatx4_t *>(slds)[i] = src[i];
+    __syncthreads();
+  }
 
   // ---- global -> register staging ---------------------------------------------------------
   // Two register sets: while the matrix cores work on the tile in LDS buffer (s & 1), set (s+1)&1
@@ -262,7 +291,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
   auto load_w = [&](auto set_, int t) {
     constexpr int set = decltype(set_)::value;
     const int64_t r0 = tile_r0(t);
-    if constexpr (!kInt4) {
+    if constexpr (!kInt4 && !kSLds) {
       if (g.scale_mode == SM_VEC4) {
         constexpr int rows = kBackward ? 4 : 2;
         constexpr int quads = kBackward ? 2 : 4;
@@ -312,10 +341,21 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
     }
   };
   // int8: fp32 value of 4 codes of dword p whose first code has flat index f
+  // the four scales of code dword `slot` of register row `row` (quads of a row are 4 apart)
+  auto scale_quad = [&](auto set_, int row, int quad, int slot) {
+    constexpr int set = decltype(set_)::value;
+    if constexpr (kSLds) {
+      uint32_t idx = sidx[row] + 4 * quad;
+      if (idx >= period32) idx -= period32;
+      return *reinterpret_cast<const floatx4_t *>(slds + idx);
+    } else {
+      return wsc8[set][slot];
+    }
+  };
   auto deq8 = [&](uint32_t p, const floatx4_t &s, int64_t f, float (&out)[4]) {
     float q[4];
     int8x4_to_f32(p, q);
-    if (g.scale_mode == SM_VEC4) {
+    if (kSLds || g.scale_mode == SM_VEC4) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) out[j] = q[j] * s[j];
     } else {
@@ -342,8 +382,8 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
         const int i = part >> 1;
         const int j = part & 1;
         float lo[4], hi[4];
-        deq8(wreg[set][4 * i + 2 * j], wsc8[set][4 * i + 2 * j], w_flat[i] + r0 + 8 * j, lo);
-        deq8(wreg[set][4 * i + 2 * j + 1], wsc8[set][4 * i + 2 * j + 1], w_flat[i] + r0 + 8 * j + 4, hi);
+        deq8(wreg[set][4 * i + 2 * j], scale_quad(set_, i, 2 * j, 4 * i + 2 * j), w_flat[i] + r0 + 8 * j, lo);
+        deq8(wreg[set][4 * i + 2 * j + 1], scale_quad(set_, i, 2 * j + 1, 4 * i + 2 * j + 1), w_flat[i] + r0 + 8 * j + 4, hi);
         u32x4_t v;
         v[0] = pack2<CT>(lo[0], lo[1]);
         v[1] = pack2<CT>(lo[2], lo[3]);
@@ -358,8 +398,8 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
       } else {
         const int64_t f = w_flat[i] + r0 * g.K;
         float lo[4], hi[4];
-        deq8(wreg[set][2 * i], wsc8[set][2 * i], f, lo);
-        deq8(wreg[set][2 * i + 1], wsc8[set][2 * i + 1], f + 4, hi);
+        deq8(wreg[set][2 * i], scale_quad(set_, i, 0, 2 * i), f, lo);
+        deq8(wreg[set][2 * i + 1], scale_quad(set_, i, 1, 2 * i + 1), f + 4, hi);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           et[i][j] = lo[j];
@@ -374,6 +414,15 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
           v[0] = pack2<CT>(et[0][j], et[1][j]);
           v[1] = pack2<CT>(et[2][j], et[3][j]);
           *reinterpret_cast<u32x2_t *>(dst + swz(wf_c + j, wf_r >> 3) + ((wf_r & 4) << 1)) = v;
+        }
+      }
+    }
+    if constexpr (!kInt4 && kSLds) {
+      if (part == 3) {        // tiles are stored in order: move every row's scale position to the next tile
+#pragma unroll
+        for (int i = 0; i < (kBackward ? 4 : 2); ++i) {
+          sidx[i] += g.scale_step;
+          if (sidx[i] >= period32) sidx[i] -= period32;
         }
       }
     }
@@ -497,19 +546,19 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(TileArgs g)
   }
 }
 
-template <typename CT, typename XT, bool kInt4, bool kBackward, bool kGrouped, int BM>
+template <typename CT, typename XT, bool kInt4, bool kSLds, bool kBackward, bool kGrouped, int BM>
 int launch_one(const TileArgs &t, int64_t row_tiles, hipStream_t s)
 {
   const int64_t C = kBackward ? t.K : t.N;
-  constexpr size_t lds = 2 * (static_cast<size_t>(BM) * BR * 2 + kBTileBytes);
-  auto kern = qgemm_kernel<CT, XT, kInt4, kBackward, kGrouped, BM>;
+  const size_t lds = 2 * (static_cast<size_t>(BM) * BR * 2 + kBTileBytes) + (kSLds ? static_cast<size_t>(t.period) * 4 : 0);
+  auto kern = qgemm_kernel<CT, XT, kInt4, kSLds, kBackward, kGrouped, BM>;
   if (lds > 64 * 1024) {
-    static bool raised = false;
-    if (!raised) {
+    static size_t raised = 0;      // largest dynamic LDS size this kernel has been enabled for
+    if (lds > raised) {
       if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                               static_cast<int>(lds)) != hipSuccess)
         return CAIFX_ERR_LAUNCH_FAILED;
-      raised = true;
+      raised = lds;
     }
   }
   const int64_t col_tiles = (C + BC - 1) / BC;
@@ -523,6 +572,22 @@ int launch_one(const TileArgs &t, int64_t row_tiles, hipStream_t s)
   return launch_status();
 }
 
+// int8 scale vectors up to this many entries are kept in LDS: 8 KiB next to the 64 KiB of a
+// 128-row workgroup leaves room for two workgroups per compute unit, 56 KiB next to the 96 KiB of
+// a 256-row workgroup fills the 160 KiB of one.
+constexpr int64_t kSLdsMax128 = 2048;
+constexpr int64_t kSLdsMax256 = 14336;
+
+template <typename CT, typename XT, bool kInt4, bool kBackward, bool kGrouped, int BM>
+int launch_scales(const TileArgs &t, int64_t row_tiles, hipStream_t s)
+{
+  if constexpr (!kInt4) {
+    if (t.scale_mode == SM_VEC4 && t.period <= (BM == 128 ? kSLdsMax128 : kSLdsMax256))
+      return launch_one<CT, XT, false, true, kBackward, kGrouped, BM>(t, row_tiles, s);
+  }
+  return launch_one<CT, XT, kInt4, false, kBackward, kGrouped, BM>(t, row_tiles, s);
+}
+
 // Tile height.  LDS bandwidth (128 B/clk per CU) is what bounds this kernel: a consumer wave reads
 // one 16-byte fragment per lane for every 32x32x16 MFMA it feeds, and with 64x64 wave tiles that is
 // one fragment read per MFMA.  256-row workgroup tiles (128x64 per consumer wave) need 0.75 reads
@@ -534,15 +599,23 @@ int launch_tile(const TileArgs &t, bool grouped, hipStream_t s)
   const int64_t C = kBackward ? t.K : t.N;
   const int64_t col_tiles = (C + BC - 1) / BC;
   if (grouped) {
-    const int64_t row_tiles = (t.M + 127) / 128 + t.num_experts;   // every expert can add one partial tile
+    // Segment lengths live on the device; the host only knows their mean.  A 256-row tile does twice
+    // the work of a 128-row tile in about the same time (the staging of the weight piece is what a
+    // step costs), so it wins whenever segments are long enough to fill most of it.  Only the int4
+    // forward kernel is lean enough in registers to keep two 128-row workgroups per compute unit,
+    // which makes up for that.
+    const bool tall_tiles = t.M / t.num_experts > 160 && (!kInt4 || kBackward);
+    const int bm = tall_tiles ? 256 : 128;
+    const int64_t row_tiles = (t.M + bm - 1) / bm + t.num_experts;   // every expert can add one partial tile
     if (row_tiles > 65535) return CAIFX_ERR_UNSUPPORTED;
-    return launch_one<CT, XT, kInt4, kBackward, true, 128>(t, row_tiles, s);
+    if (tall_tiles) return launch_scales<CT, XT, kInt4, kBackward, true, 256>(t, row_tiles, s);
+    return launch_scales<CT, XT, kInt4, kBackward, true, 128>(t, row_tiles, s);
   }
   const int64_t tall = (t.M + 255) / 256;
-  if (tall * col_tiles >= 200 && tall <= 65535) return launch_one<CT, XT, kInt4, kBackward, false, 256>(t, tall, s);
+  if (tall * col_tiles >= 200 && tall <= 65535) return launch_scales<CT, XT, kInt4, kBackward, false, 256>(t, tall, s);
   const int64_t row_tiles = (t.M + 127) / 128;
   if (row_tiles > 65535) return CAIFX_ERR_UNSUPPORTED;
-  return launch_one<CT, XT, kInt4, kBackward, false, 128>(t, row_tiles, s);
+  return launch_scales<CT, XT, kInt4, kBackward, false, 128>(t, row_tiles, s);
 }
 
 template <typename CT, typename XT>

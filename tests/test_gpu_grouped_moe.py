@@ -41,6 +41,41 @@ def test_grouped_forward_backward_segments(orc, kind):
     assert not y[total:].any() and not dx[total:].any()
 
 
+def _check_segments(orc, rng, counts, N, K, kind, group=128):
+    E = len(counts)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    total = int(offsets[-1])
+    ows, gw = _experts(orc, rng, E, N, K, kind, group)
+    x = dev_as(rng.normal(0, 1, (total, K)), 2)
+    dy = dev_as(rng.normal(0, 1e-2, (total, N)), 2)
+    off_d = dev(offsets)
+    y = host(T.qlinear_grouped_forward(x, off_d, gw, 2))
+    dx = host(T.qlinear_grouped_backward_input(dy, off_d, gw, 2))
+    xh, dyh = host(x), host(dy)
+    for e in range(E):
+        lo, hi = offsets[e], offsets[e + 1]
+        if hi == lo:
+            continue
+        assert max_rel_err(y[lo:hi], orc.frozen_linear_forward(xh[lo:hi], ows[e], 2)) <= 5e-5, (kind, e)
+        assert max_rel_err(dx[lo:hi], orc.frozen_linear_backward(dyh[lo:hi], ows[e], 2)) <= 5e-5, (kind, e)
+
+
+@pytest.mark.parametrize("kind", ["int8pc", "int4", "int8pt"])
+def test_grouped_long_segments_take_tall_tiles(orc, kind):
+    # a mean of more than 160 rows per expert switches the int8 kernels and the int4 input gradient
+    # to 256-row tiles: full tiles, a partial last tile, an empty expert
+    _check_segments(orc, np.random.default_rng(11), np.array([300, 0, 517, 256]), 192, 256, kind)
+
+
+def test_grouped_more_experts_than_lanes(orc):
+    # 70 experts: the tile -> expert search runs over more than one 64-lane chunk of the offsets
+    rng = np.random.default_rng(12)
+    counts = rng.integers(0, 40, 70)
+    counts[[0, 63, 64, 69]] = [0, 129, 7, 33]
+    _check_segments(orc, rng, counts, 128, 128, "int8pc")
+    _check_segments(orc, rng, counts, 128, 128, "int4", group=32)
+
+
 def test_grouped_equals_per_expert_calls(orc):
     rng = np.random.default_rng(2)
     E, N, K = 4, 256, 128
