@@ -6,17 +6,21 @@
 // with B drawn from the stored weight W[N,K]:
 //     forward : C = N, R = K, B[r][c] = W[c][r]   (a weight row is contiguous along R)
 //     backward: C = K, R = N, B[r][c] = W[r][c]   (a weight row is contiguous along C)
-// A workgroup (512 threads: 2x2 consumer waves that run the MFMAs + 4 producer waves that stage the
-// operands) owns a BM x 128 tile of D (BM = 128 is what is launched) and walks R in steps of 64.
-// Per step it moves a BMx64 tile of A and the matching 64x128 piece of W from global memory
-// into registers two steps ahead of their use, dequantises W in
-// registers (code * scale in fp32, one rounding to the compute dtype: bit-identical to the
-// reference's dequantise-then-cast weight) and writes both tiles to the other half of a
-// double-buffered LDS area, as [row][64 values along R] with the 16-byte chunks of a row
-// XOR-swizzled by (row & 7) so that the 128-bit operand reads of v_mfma_f32_32x32x16 spread
-// over all banks.  For the backward case the weight piece is transposed on the way: a thread
-// holds 4 weight rows x 8 columns and writes 8 runs of 4 values along R.
-// Each wave accumulates a (BM/2) x 64 sub-tile (64 or 128 fp32 accumulators per lane).
+// A workgroup of 512 threads owns a BM x 128 tile of D (BM = 256 when that still gives enough
+// tiles to fill the chip, else 128) and walks R in steps of 64.  Its waves are specialised: waves
+// 4..7 ("producers") stage operands, waves 0..3 ("consumers", laid out 2x2 over the tile) run the
+// MFMAs, one of each per SIMD, so unpacking arithmetic and the matrix pipe overlap without any
+// instruction-level interleaving.  Per step the producers move a BMx64 tile of A and the matching
+// 64x128 piece of W from global memory into registers two steps ahead of their use, dequantise W
+// there (code * scale in fp32, one rounding to the compute dtype: bit-identical to the reference's
+// dequantise-then-cast weight) and write both tiles to the other half of a double-buffered LDS
+// area, as [row][64 values along R] with the 16-byte chunks of a row XOR-swizzled by row bits so
+// that the 128-bit operand reads of v_mfma_f32_32x32x16 and the transposed writes of the backward
+// case spread over all banks.  For the backward case the weight piece is transposed on the way:
+// a thread holds 4 weight rows x 8 columns and writes 8 runs of 4 values along R.
+// A consumer wave accumulates a (BM/2) x 64 sub-tile (64 or 128 fp32 accumulators per lane) and
+// keeps the operand fragments of the next 16-wide k step in flight while the MFMAs of the current
+// one issue.  All eight waves meet at one barrier per step.
 // No dense copy of W ever reaches HBM; the only HBM traffic is A, the packed W and D.
 #include "caifx_internal.hpp"
 
@@ -588,11 +592,10 @@ int launch_scales(const TileArgs &t, int64_t row_tiles, hipStream_t s)
   return launch_one<CT, XT, kInt4, false, kBackward, kGrouped, BM>(t, row_tiles, s);
 }
 
-// Tile height.  LDS bandwidth (128 B/clk per CU) is what bounds this kernel: a consumer wave reads
-// one 16-byte fragment per lane for every 32x32x16 MFMA it feeds, and with 64x64 wave tiles that is
-// one fragment read per MFMA.  256-row workgroup tiles (128x64 per consumer wave) need 0.75 reads
-// per MFMA and half the weight staging per flop, so they are used whenever there are enough of
-// them to fill the chip; expert segments (a few hundred rows each) keep 128-row tiles.
+// Tile height.  What a step costs is mostly the staging chain of the producers, and a 256-row
+// tile stages the same 64x128 weight piece as a 128-row tile for twice the MFMA work; its consumer
+// waves (128x64 each) also need only 0.75 operand-fragment reads per MFMA instead of 1.  So
+// 256-row tiles are used whenever there are enough of them to fill the chip.
 template <typename CT, typename XT, bool kInt4, bool kBackward>
 int launch_tile(const TileArgs &t, bool grouped, hipStream_t s)
 {
