@@ -31,8 +31,7 @@ namespace {
 
 constexpr int BC = 128;      // columns of D per workgroup
 constexpr int BR = 64;       // reduction extent per step
-constexpr int kStagers = 256;               // producer threads (stage A and W tiles into LDS)
-constexpr int kThreads = 512;               // 4 consumer waves (MFMA) + 4 producer waves
+constexpr int kWStagers = 256;              // producer threads that stage the W piece (the first four producer waves)
 constexpr int kBTileBytes = BC * BR * 2;   // weight tile in LDS (16 KiB)
 
 template <typename CT> struct Mfma32;
@@ -95,22 +94,27 @@ __device__ __forceinline__ float int8_scale_at(const float *scales, int mode, in
 // kSLds (int8 with a periodic scale vector that fits): the scale vector sits in LDS behind the
 // tile buffers and is read when a weight piece is dequantised, instead of travelling through
 // registers with the codes.
-template <typename CT, typename XT, bool kInt4, bool kSLds, bool kBackward, bool kGrouped, int BM>
-__global__ __launch_bounds__(kThreads, (BM == 128 && (kInt4 || kSLds)) ? 4 : 2) void qgemm_kernel(TileArgs g)
+// kCW: consumer waves (4 or 8), laid out (kCW/2) x 2 over the tile; there are as many producer waves.
+template <typename CT, typename XT, bool kInt4, bool kSLds, bool kBackward, bool kGrouped, int BM, int kCW>
+__global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || kSLds))) ? 4 : 2) void qgemm_kernel(TileArgs g)
 {
+  constexpr int kThreads = 2 * kCW * 64;
+  constexpr int kStagers = kCW * 64;                         // producer threads
+  constexpr int kWaveRows = BM / (kCW / 2);                  // rows of D per consumer wave
   typedef typename Mfma32<CT>::vec_t vec_t;
   constexpr int kATileBytes = BM * BR * 2;
   constexpr int kAStages = 2;
   constexpr int kBBase = kAStages * kATileBytes;             // LDS: A ring, then two B buffers
   constexpr int kSBase = kBBase + 2 * kBTileBytes;           // ... then the int8 scale vector (kSLds)
-  constexpr int WR = BM / 64;                                // 32-row MFMA tiles per wave along M
-  constexpr int kAChunks = BM / 32;                          // 16-byte LDS chunks of A per thread per step
+  constexpr int WR = kWaveRows / 32;                         // 32-row MFMA tiles per wave along M
+  constexpr int kAChunks = BM * 8 / kStagers;                // 16-byte LDS chunks of A per thread per step
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];          // 2 x kStageBytes
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const bool producer = wave >= 4;                 // waves 4..7 stage tiles, waves 0..3 run the MFMAs
-  const int tid = threadIdx.x & (kStagers - 1);    // staging thread index (producers)
-  const int wm = (wave >> 1) & 1;  // consumer wave row (0..1): BM/2 rows of D
+  const bool producer = wave >= kCW;               // the upper half of the waves stages tiles, the lower half runs the MFMAs
+  const int tid = threadIdx.x - kStagers;          // staging thread index (producers)
+  const bool w_stager = tid < kWStagers;           // wave-uniform: the W piece is laid out for 256 threads
+  const int wm = wave >> 1;        // consumer wave row: kWaveRows rows of D
   const int wc = wave & 1;         // consumer wave column (0..1): 64 columns of D
 
   const int64_t R = kBackward ? g.N : g.K;     // reduction length
@@ -208,10 +212,14 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (kInt4 || kSLds)) ? 4 : 2) 
     if (m >= row_hi) m = row_hi - 1;                    // clamp: rows past the end are never stored
     a_ptr[i] = ag + m * R + (q & 7) * 8;
   }
-  auto load_a = [&](auto set_, int64_t r0) {
+  // part < 0: the whole tile; else the quarter of this thread's chunks that store_a(part) has just
+  // written out, so that the requests spread over the step instead of queueing up at its end
+  auto load_a = [&](auto set_, int64_t r0, int part = -1) {
     constexpr int set = decltype(set_)::value;
+    constexpr int per = kAChunks / 4;
 #pragma unroll
     for (int i = 0; i < kAChunks; ++i) {
+      if (part >= 0 && i / per != part) continue;
       if constexpr (sizeof(XT) == 4) {
         areg[set][2 * i] = *reinterpret_cast<const u32x4_t *>(a_ptr[i] + r0);
         areg[set][2 * i + 1] = *reinterpret_cast<const u32x4_t *>(a_ptr[i] + r0 + 4);
@@ -443,30 +451,33 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (kInt4 || kSLds)) ? 4 : 2) 
 
   if (producer) {
     load_a(I0{}, 0);
-    load_w(I0{}, 0);
+    if (w_stager) load_w(I0{}, 0);
 #pragma unroll
     for (int part = 0; part < 4; ++part) {
       store_a(I0{}, smem, part);
-      store_w(I0{}, smem + kBBase, 0, part);
+      if (w_stager) store_w(I0{}, smem + kBBase, 0, part);
     }
     load_a(I1{}, tile_r0(1));
-    load_w(I1{}, 1);
+    if (w_stager) load_w(I1{}, 1);
     load_a(I0{}, tile_r0(2));
-    load_w(I0{}, 2);
+    if (w_stager) load_w(I0{}, 2);
     __syncthreads();
     // step s: register set (s+1)&1 holds tile s+1 -> LDS buffer (s+1)&1, then that set <- tile s+3
-    // (set p always carries tiles of parity p; a load has two steps to arrive)
+    // (set p always carries tiles of parity p; a load has two steps to arrive).  The A chunks are
+    // requested again right after they have been written out, so that the requests spread over the
+    // step instead of queueing up at its end.
     auto pstep = [&](auto buf_, int s) {
       constexpr int buf = decltype(buf_)::value;
       typedef std::integral_constant<int, 1 - buf> NxtSet;
       const int64_t r_next = tile_r0(s + 1);
+      const int64_t r_load = tile_r0(s + 3);
 #pragma unroll
       for (int part = 0; part < 4; ++part) {
         store_a(NxtSet{}, smem + (1 - buf) * kATileBytes, part);
-        store_w(NxtSet{}, smem + kBBase + (1 - buf) * kBTileBytes, r_next, part);
+        load_a(NxtSet{}, r_load, part);
+        if (w_stager) store_w(NxtSet{}, smem + kBBase + (1 - buf) * kBTileBytes, r_next, part);
       }
-      load_a(NxtSet{}, tile_r0(s + 3));
-      load_w(NxtSet{}, s + 3);
+      if (w_stager) load_w(NxtSet{}, s + 3);
       __syncthreads();
     };
     int s = 0;
@@ -501,7 +512,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (kInt4 || kSLds)) ? 4 : 2) 
     auto read_frags = [&](int fb, int ks) {
 #pragma unroll
       for (int i = 0; i < WR; ++i)
-        af[fb][i] = *reinterpret_cast<const vec_t *>(abuf + swz(wm * (BM / 2) + i * 32 + frow, ks * 2 + fh));
+        af[fb][i] = *reinterpret_cast<const vec_t *>(abuf + swz(wm * kWaveRows + i * 32 + frow, ks * 2 + fh));
 #pragma unroll
       for (int j = 0; j < 2; ++j)
         bf[fb][j] = *reinterpret_cast<const vec_t *>(bbuf + swz(wc * 64 + j * 32 + frow, ks * 2 + fh));
@@ -536,7 +547,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (kInt4 || kSLds)) ? 4 : 2) 
       if (col < C) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int64_t row = row_lo + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          const int64_t row = row_lo + wm * kWaveRows + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
           if (row < row_hi) {
             const int64_t o = row * C + col;
             const float v = acc[i][j][r];
@@ -550,12 +561,13 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (kInt4 || kSLds)) ? 4 : 2) 
   }
 }
 
-template <typename CT, typename XT, bool kInt4, bool kSLds, bool kBackward, bool kGrouped, int BM>
+template <typename CT, typename XT, bool kInt4, bool kSLds, bool kBackward, bool kGrouped, int BM, int kCW = 4>
 int launch_one(const TileArgs &t, int64_t row_tiles, hipStream_t s)
 {
+  constexpr int kThreads = 2 * kCW * 64;
   const int64_t C = kBackward ? t.K : t.N;
   const size_t lds = 2 * (static_cast<size_t>(BM) * BR * 2 + kBTileBytes) + (kSLds ? static_cast<size_t>(t.period) * 4 : 0);
-  auto kern = qgemm_kernel<CT, XT, kInt4, kSLds, kBackward, kGrouped, BM>;
+  auto kern = qgemm_kernel<CT, XT, kInt4, kSLds, kBackward, kGrouped, BM, kCW>;
   if (lds > 64 * 1024) {
     static size_t raised = 0;      // largest dynamic LDS size this kernel has been enabled for
     if (lds > raised) {
