@@ -159,7 +159,7 @@ def main():
     dom = ("int8", 1)           # the kernel that takes most of a step
     roofline = {
         "bound": "hbm",
-        "kernel": "rowlin_int8_fast_kernel<bf16, 1 row, per-channel scales, 4 chunks/row> M=1 K=4096 N=14336",
+        "kernel": "rowlin_int8_digits_kernel<bf16 X, per-channel scales, 4 chunks/row> M=1 K=4096 N=14336",
         "achieved": round(per[dom]["GBps"], 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",

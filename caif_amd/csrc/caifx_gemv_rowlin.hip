@@ -19,10 +19,13 @@
 //     one 128-k scale group, so D[i][i] is a per-group sum of (code+136 or code+1032) * x and
 //     the lane holding it applies  scale * (D[i][i] - offset * sum_k x)  -- the post-scaled form
 //     (see caifx_gemv.hip for the numerics note).
-//   int8: a k-slot is 16 codes; float(code)*scale is rounded to the compute dtype exactly as
-//     the reference does.  With per-channel scales the index (n*K+k) % period depends on the
+//   int8 (two to four activation rows, and one row when the shape does not fit the kernel below):
+//     a k-slot is 16 codes; float(code)*scale is rounded to the compute dtype exactly as the
+//     reference does.  With per-channel scales the index (n*K+k) % period depends on the
 //     row only through (n*K) % period, so a wave takes rows of one residue class
 //     n = v + V*i (V = period / gcd(K, period)) and keeps that class's scales in registers.
+//   int8, one activation row, K a multiple of 1024: the scales are folded into the activations and
+//     the codes go into the integer matrix core as loaded (rowlin_int8_digits_kernel below).
 #include "caifx_internal.hpp"
 
 namespace caifx {
@@ -64,6 +67,7 @@ struct RowArgs {
   int total_waves;
   int cpr;              // chunks (one load instruction of a wave) per weight row
   int xpitch;           // staged activations: elements per row (cpr * k-per-chunk)
+  int digits;           // int8, one activation row: take the integer-matrix-core kernel
 };
 
 template <typename CT, typename XT>
@@ -568,6 +572,166 @@ __global__ __launch_bounds__(256) void rowlin_int8_fast_kernel(RowArgs a)
   }
 }
 
+// ------------------------------------------------------------------ int8, one activation row, integer matrix core
+// Y[n] = sum_k q[n,k] * scale[(n*K+k) mod P] * x[k].  All rows of one residue class see the same
+// scales along k, so the scales are folded into the activations once per workgroup:
+// x'[k] = scale[(cls*K+k) mod P] * x[k] (fp32), and x' is split into three signed 7-bit "digits"
+// relative to a power-of-two scale per diagonal element (the 256 k values of lanes i, i+16, i+32,
+// i+48): x' ~ 2^(e-6) * (d0 + d1/128 + d2/16384), |error| <= 2^(e-21).  The int8 codes then go into
+// v_mfma_i32_16x16x64_i8 exactly as they were loaded (one 16-byte load = one A operand, no
+// unpacking arithmetic at all) against the digit planes as B operands; the three int32 sums are exact
+// and are combined in fp32 once per weight row.  As in the kernels above only the diagonal of the
+// 16x16 result is used.  The result is sum_k q*scale*x with every product exact to ~2^-21 of the
+// largest |x'| of its 256-k set; it differs from the reference's dequantise-round-GEMM by the rounding
+// of q*scale to the compute dtype that the reference applies and this kernel does not.
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+
+template <typename XT, bool kVec, int CPR>
+__global__ __launch_bounds__(256) void rowlin_int8_digits_kernel(RowArgs a)
+{
+  constexpr int D = (CPR >= 4) ? 1 : 4 / CPR;   // rows in flight (4 loads per lane measured best)
+  __shared__ float mx[4][16];                                  // per chunk: max |x'| of every diagonal element
+  __shared__ __attribute__((aligned(16))) i32x4_t dig[4][3][64];   // [chunk][digit][lane]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int gw = blockIdx.x * 4 + wave;
+  const int cls = (blockIdx.x * 4) / a.waves_per_class;        // waves_per_class is a multiple of 4: one class per workgroup
+  const int64_t i0 = static_cast<int64_t>(gw - cls * a.waves_per_class) * a.rows_per_wave;
+  const int64_t V = a.row_stride;
+  int nrows = 0;
+  {
+    const int64_t first = cls + V * i0;
+    if (first < a.N) {
+      const int64_t avail = (a.N - first + V - 1) / V;
+      nrows = static_cast<int>(avail < a.rows_per_wave ? avail : a.rows_per_wave);
+    }
+  }
+  constexpr int64_t kRowBytes = static_cast<int64_t>(CPR) * 1024;
+
+  // this lane's activations of chunk `wave` (chunks beyond CPR do not exist; their waves only join the barriers)
+  float xv[16];
+  const bool has_chunk = wave < CPR;
+  if (has_chunk) {
+    const XT *xg = static_cast<const XT *>(a.x) + (wave * 64 + lane) * 16;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) xv[t] = to_f32<XT>(xg[t]);
+  }
+
+  const uint8_t *wp = a.wq + (cls + V * i0) * kRowBytes + lane * 16;
+  const int64_t rstep = V * kRowBytes;
+  i32x4_t w[D][CPR];
+  auto issue = [&](int d, int r) {
+#pragma unroll
+    for (int c = 0; c < CPR; ++c) w[d][c] = *reinterpret_cast<const i32x4_t *>(wp + r * rstep + c * 1024);
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < nrows) issue(d, d);
+
+  float s_scalar = 1.0f;
+  if (has_chunk) {
+    if constexpr (kVec) {
+      const float *sp = static_cast<const float *>(a.scales);
+      const int idx = static_cast<int>((static_cast<int64_t>(cls) * (CPR * 1024) + (wave * 64 + lane) * 16) % a.period);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        int i = idx + 4 * q;
+        if (i >= a.period) i -= a.period;
+        const floatx4_t sc = *reinterpret_cast<const floatx4_t *>(sp + i);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) xv[4 * q + t] *= sc[t];
+      }
+    }
+    float m = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) m = fmaxf(m, fabsf(xv[t]));
+    m = fmaxf(m, __shfl_xor(m, 16));
+    m = fmaxf(m, __shfl_xor(m, 32));
+    if (lane < 16) mx[wave][lane] = m;
+  }
+  if constexpr (!kVec) {
+    if (a.scales) s_scalar = static_cast<const float *>(a.scales)[0];
+  }
+  __syncthreads();
+
+  // power-of-two unit of diagonal element i: the largest |x'| of its CPR*64 values maps into [32, 64]
+  float unit;
+  {
+    float m = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CPR; ++c) m = fmaxf(m, mx[c][lane & 15]);
+    int e = 0;
+    (void)frexpf(m, &e);                      // m = f * 2^e, f in [0.5, 1)
+    unit = m > 0.0f ? ldexpf(1.0f, e - 6) : 1.0f;
+  }
+  if (has_chunk) {
+    const float inv = 1.0f / unit;            // exact: a power of two
+    i32x4_t d0, d1, d2;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      uint32_t b0 = 0, b1 = 0, b2 = 0;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const float v = xv[4 * q + t] * inv;           // |v| <= 64
+        const float r0 = rintf(v);
+        const float v1 = (v - r0) * 128.0f;            // exact, |v1| <= 64
+        const float r1 = rintf(v1);
+        const float r2 = rintf((v1 - r1) * 128.0f);
+        b0 |= (static_cast<uint32_t>(static_cast<int>(r0)) & 0xFFu) << (8 * t);
+        b1 |= (static_cast<uint32_t>(static_cast<int>(r1)) & 0xFFu) << (8 * t);
+        b2 |= (static_cast<uint32_t>(static_cast<int>(r2)) & 0xFFu) << (8 * t);
+      }
+      d0[q] = static_cast<int>(b0);
+      d1[q] = static_cast<int>(b1);
+      d2[q] = static_cast<int>(b2);
+    }
+    dig[wave][0][lane] = d0;
+    dig[wave][1][lane] = d1;
+    dig[wave][2][lane] = d2;
+  }
+  __syncthreads();
+  i32x4_t xb[CPR][3];
+#pragma unroll
+  for (int c = 0; c < CPR; ++c)
+#pragma unroll
+    for (int d = 0; d < 3; ++d) xb[c][d] = dig[c][d][lane];
+  const float u0 = unit * s_scalar, u1 = u0 * (1.0f / 128.0f), u2 = u0 * (1.0f / 16384.0f);
+  const int tsel = lane & 3;
+  const bool is_diag = (lane >> 4) == ((lane & 15) >> 2);
+
+  for (int r0 = 0; r0 < nrows; r0 += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int r = r0 + d;
+      if (r < nrows) {
+        i32x4_t wr[CPR];
+#pragma unroll
+        for (int c = 0; c < CPR; ++c) wr[c] = w[d][c];
+        if (r + D < nrows) issue(d, r + D);
+        i32x4_t s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0}, s2 = {0, 0, 0, 0};
+#pragma unroll
+        for (int c = 0; c < CPR; ++c) {
+          s0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[c], xb[c][0], s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[c], xb[c][1], s1, 0, 0, 0);
+          s2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[c], xb[c][2], s2, 0, 0, 0);
+        }
+        // D[i][i] sits in element i%4 of lane i + 16*(i/4)
+        int p0 = s0[0], p1 = s1[0], p2 = s2[0];
+        p0 = tsel == 1 ? s0[1] : p0;  p1 = tsel == 1 ? s1[1] : p1;  p2 = tsel == 1 ? s2[1] : p2;
+        p0 = tsel == 2 ? s0[2] : p0;  p1 = tsel == 2 ? s1[2] : p1;  p2 = tsel == 2 ? s2[2] : p2;
+        p0 = tsel == 3 ? s0[3] : p0;  p1 = tsel == 3 ? s1[3] : p1;  p2 = tsel == 3 ? s2[3] : p2;
+        float v = static_cast<float>(p0) * u0;
+        v = __builtin_fmaf(static_cast<float>(p1), u1, v);
+        v = __builtin_fmaf(static_cast<float>(p2), u2, v);
+        v = wave_sum_hi(is_diag ? v : 0.0f);
+        if (lane == 63) static_cast<float *>(a.y)[cls + V * (i0 + r)] = v;
+      }
+    }
+  }
+}
+
+
 // ------------------------------------------------------------------ int8, exact
 // kVec: per-channel scales (period > 1) cached in registers per residue class.
 template <typename CT, typename XT, int MT, bool kVec, int CPR>
@@ -713,9 +877,23 @@ int launch_int4(const RowArgs &ra, hipStream_t s)
   return launch_status();
 }
 
+template <typename XT, bool kVec, int CPR>
+int launch_int8_digits(const RowArgs &ra, hipStream_t s)
+{
+  hipLaunchKernelGGL((rowlin_int8_digits_kernel<XT, kVec, CPR>), dim3(static_cast<unsigned>(ra.total_waves / 4)), dim3(256), 0, s, ra);
+  return launch_status();
+}
+
 template <typename CT, typename XT, int MT, bool kVec>
 int launch_int8(const RowArgs &ra, hipStream_t s)
 {
+  if constexpr (MT == 1) {
+    if (ra.digits) {
+      if (ra.cpr == 1) return launch_int8_digits<XT, kVec, 1>(ra, s);
+      if (ra.cpr == 2) return launch_int8_digits<XT, kVec, 2>(ra, s);
+      return launch_int8_digits<XT, kVec, 4>(ra, s);
+    }
+  }
   if constexpr (dtype_code<XT>::value == dtype_code<CT>::value) {
     const bool full = (ra.K % 1024 == 0) && ra.y_dtype == CAIFX_F32;
     if (full && ra.cpr == 1) return launch_int8_fast<CT, MT, kVec, 1>(ra, s);
@@ -770,11 +948,11 @@ int64_t gcd64(int64_t a, int64_t b)
   return a;
 }
 
-int pick_rows_per_wave(int64_t rows, int min_rows)
+int pick_rows_per_wave(int64_t rows, int min_rows, int64_t target = 2048)
 {
   // aim for two waves per SIMD (2048 waves): each walks its rows through a ring of loads, so
   // unpacking overlaps the HBM latency of the rows behind it
-  int64_t rpw = (rows + 2047) / 2048;
+  int64_t rpw = (rows + target - 1) / target;
   if (rpw < min_rows) rpw = min_rows;
   if (rpw > 64) rpw = 64;
   return static_cast<int>(rpw);
@@ -829,8 +1007,14 @@ int rowlin_forward(const GemmArgs &g, hipStream_t s)
     }
     const int64_t rows_class = (g.N + ra.row_stride - 1) / ra.row_stride;
     const int rb = ra.cpr == 1 ? 8 : (ra.cpr == 2 ? 4 : 2);
-    ra.rows_per_wave = pick_rows_per_wave(g.N, kind == 2 ? 2 * rb : rb);
+    const bool digits = g.M == 1 && g.K % 1024 == 0 && (ra.cpr == 1 || ra.cpr == 2 || ra.cpr == 4) && g.y_dtype == CAIFX_F32;
+    // the integer-matrix-core kernel is light on registers and arithmetic: four waves per SIMD measured best
+    ra.rows_per_wave = digits ? pick_rows_per_wave(g.N, 1, 4096) : pick_rows_per_wave(g.N, kind == 2 ? 2 * rb : rb);
     ra.waves_per_class = static_cast<int>((rows_class + ra.rows_per_wave - 1) / ra.rows_per_wave);
+    if (digits) {
+      ra.digits = 1;
+      ra.waves_per_class = (ra.waves_per_class + 3) / 4 * 4;      // a workgroup of 4 waves stays inside one class
+    }
     ra.total_waves = ra.waves_per_class * ra.row_stride;
     if (static_cast<size_t>(mt) * ra.xpitch * 2 > 64 * 1024) return CAIFX_ERR_UNSUPPORTED;
   }

@@ -3,11 +3,13 @@
 Tolerance (north star): max relative error <= 1e-2 for bf16/fp16 compute with fp32
 accumulation, <= 1e-4 for the fp32 path; both relative to max|ref| as the reference's own
 parity tests normalise.  The asserts are tighter than the contract:
-  * int8 and int4 with group sizes below 128 feed the matrix cores weights that are
-    bit-identical to the oracle's, so only the summation order differs (~1e-6);
-  * int4 with group size 128 (or a multiple) is scaled after the per-group accumulation, which
-    skips the reference's bf16 rounding of code*scale: the difference is that rounding,
-    <= 2^-9 per weight with random sign, a few 1e-4 of max|ref| after the sum over K.
+  * int8 (two rows and more) and int4 with group sizes below 128 feed the matrix cores weights
+    that are bit-identical to the oracle's, so only the summation order differs (~1e-6);
+  * int4 with group size 128 (or a multiple) is scaled after the per-group accumulation, and int8
+    with one activation row and K a multiple of 1024 folds the scales into the activations and
+    multiplies integer codes exactly: both skip the reference's rounding of code*scale to the
+    compute dtype; the difference is that rounding, <= 2^-9 per weight with random sign, about
+    2e-3 of max|ref| after the sum over K.
 """
 import numpy as np
 import pytest
@@ -35,7 +37,7 @@ def _check(orc, rng, M, N, K, kind, cd, xd, group=128, yd=0):
     bound = TOL_32 if cd == 0 else TOL_16
     assert err <= bound, (M, N, K, kind, cd, xd, err)
     if cd != 0 and yd == 0:
-        post = kind == "int4" and group % 128 == 0
+        post = (kind == "int4" and group % 128 == 0) or (kind.startswith("int8") and M == 1 and K in (1024, 2048, 4096))
         assert err <= (TIGHT_POST if post else TIGHT_16), (M, N, K, kind, cd, xd, err)
     return err
 
@@ -100,13 +102,27 @@ def test_m1_equals_row0_of_m16(orc):
 
 
 def test_one_hot_reads_a_weight_column_exactly(orc):
-    # X = e_j  =>  Y[0, n] = W[n, j] exactly (a single non-zero product): in the compute dtype for the
-    # paths that round each weight, as the unrounded fp32 code*scale for post-scaled int4 (group 128)
+    # X = e_j  =>  Y[0, n] = W[n, j] (a single non-zero product).  Paths that round each weight to the
+    # compute dtype return that rounded weight bit for bit; post-scaled int4 (group 128) returns the
+    # unrounded fp32 code*scale bit for bit; one row of int8 on the integer matrix core (enough rows per
+    # scale-residue class: N = 2048 here, not N = 320) passes the scale through three 7-bit digits, so
+    # code*scale comes back exact to 2^-21.
     rng = np.random.default_rng(6)
-    for kind, group, wd in (("int4", 128, 0), ("int4", 64, 2), ("int8pc", 128, 2), ("int8pt", 128, 2)):
-        ow, dw = make_weight(orc, rng, 320, 1024, kind, group)
+    for kind, group, N, how in (("int4", 128, 320, "fp32"), ("int4", 64, 320, "bf16"), ("int8pc", 128, 320, "bf16"),
+                                ("int8pt", 128, 320, "digits"), ("int8pc", 128, 2048, "digits")):
+        ow, dw = make_weight(orc, rng, N, 1024, kind, group)
         for j in (0, 1, 4, 127, 128, 777, 1023):
             e = np.zeros((1, 1024), np.float32)
             e[0, j] = 1.0
             y = host(T.qlinear_forward(dev_as(e, 2), dw, 2))
-            assert np.array_equal(y[0], ow.compute_weight(wd)[:, j]), (kind, group, j)
+            if how == "digits":
+                assert np.allclose(y[0], ow.compute_weight(0)[:, j], rtol=1e-6, atol=0), (kind, group, N, j)
+            else:
+                assert np.array_equal(y[0], ow.compute_weight(0 if how == "fp32" else 2)[:, j]), (kind, group, N, j)
+        if kind.startswith("int8"):
+            # two rows take a kernel that rounds every weight to the compute dtype like the reference
+            e = np.zeros((2, 1024), np.float32)
+            e[0, 5] = e[1, 900] = 1.0
+            y = host(T.qlinear_forward(dev_as(e, 2), dw, 2))
+            w2 = ow.compute_weight(2)
+            assert np.array_equal(y[0], w2[:, 5]) and np.array_equal(y[1], w2[:, 900]), (kind, N)
