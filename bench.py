@@ -102,18 +102,18 @@ def main():
         return g
 
     def time_graph(g, launches, reps=5):
-        """Average milliseconds per launch, HIP events around graph replays (best of reps)."""
+        """Average milliseconds per launch, HIP events around graph replays (median of reps)."""
         g.replay()
         torch.cuda.synchronize()
-        best = float("inf")
+        times = []
         for _ in range(reps):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             g.replay()
             e1.record()
             torch.cuda.synchronize()
-            best = min(best, e0.elapsed_time(e1) / launches)
-        return best
+            times.append(e0.elapsed_time(e1) / launches)
+        return sorted(times)[len(times) // 2]
 
     # ---------------------------------------------------------------- the timed region: K steps
     for i in range(args.warmup):
@@ -139,7 +139,7 @@ def main():
         del src, dst
 
     # ---------------------------------------------------------------- per-kernel durations (HIP events)
-    L = 64
+    L = 128
     per = {}
     for kind, Ws, nc in (("int4", W4, copies4), ("int8", W8, copies8)):
         for m in (1, 4, 16):
@@ -296,13 +296,26 @@ def moe_rows(torch, T, dev, gen):
         return e0.elapsed_time(e1) / iters
 
     ms_f, ms_b = timed(fwd), timed(bwd)
+    # per-expert-segment efficiency: replay single segments (shortest, median, longest) of the gate
+    # projection as stand-alone dequant-GEMMs
+    order = torch.argsort(counts).tolist()
+    segments = {}
+    for label, e in (("shortest", order[0]), ("median", order[E // 2]), ("longest", order[-1])):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        xe, ye = x[lo:hi], up_o[lo:hi]
+        ms = timed(lambda: T.qlinear_forward(xe, gate.weights[e], T.BF16, T.BF16, out=ye, workspace=ws), iters=20)
+        fl = 2.0 * (hi - lo) * D * H
+        segments[label] = {"rows": hi - lo, "us": round(ms * 1e3, 2), "TFLOPs": round(fl / (ms * 1e-3) / 1e12, 1),
+                           "frac_of_mfma_peak": round(fl / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
     gemm_flops = 3 * 2.0 * rows * D * H
     return {"experts": E, "tokens": tokens, "top_k": top_k, "packed_rows": rows,
             "rows_per_expert_min_max": [int(counts.min()), int(counts.max())],
             "fwd_ms": round(ms_f, 4), "bwd_ms": round(ms_b, 4),
             "tokens_per_s_fwd_bwd": round(tokens / ((ms_f + ms_b) * 1e-3), 1),
             "grouped_gemm_TFLOPs_fwd": round(gemm_flops / (ms_f * 1e-3) / 1e12, 1),
-            "grouped_gemm_TFLOPs_bwd": round(gemm_flops / (ms_b * 1e-3) / 1e12, 1)}
+            "grouped_gemm_TFLOPs_bwd": round(gemm_flops / (ms_b * 1e-3) / 1e12, 1),
+            "grouped_frac_of_mfma_peak": round(2 * gemm_flops / ((ms_f + ms_b) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "single_segment_replay_gate_proj": segments}
 
 
 def cpu_baseline(np, q8, s8, p4, s4_bits, x_values):

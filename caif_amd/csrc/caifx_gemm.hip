@@ -24,6 +24,7 @@
 // No dense copy of W ever reaches HBM; the only HBM traffic is A, the packed W and D.
 #include "caifx_internal.hpp"
 
+#include <atomic>
 #include <type_traits>
 
 namespace caifx {
@@ -569,12 +570,16 @@ int launch_one(const TileArgs &t, int64_t row_tiles, hipStream_t s)
   const size_t lds = 2 * (static_cast<size_t>(BM) * BR * 2 + kBTileBytes) + (kSLds ? static_cast<size_t>(t.period) * 4 : 0);
   auto kern = qgemm_kernel<CT, XT, kInt4, kSLds, kBackward, kGrouped, BM, kCW>;
   if (lds > 64 * 1024) {
-    static size_t raised = 0;      // largest dynamic LDS size this kernel has been enabled for
-    if (lds > raised) {
+    // largest dynamic LDS size this kernel has been enabled for (the attribute is per kernel and sticky;
+    // two threads racing here both set it, which is harmless)
+    static std::atomic<size_t> raised{0};
+    if (lds > raised.load(std::memory_order_relaxed)) {
       if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                               static_cast<int>(lds)) != hipSuccess)
         return CAIFX_ERR_LAUNCH_FAILED;
-      raised = lds;
+      size_t seen = raised.load(std::memory_order_relaxed);
+      while (seen < lds && !raised.compare_exchange_weak(seen, lds, std::memory_order_relaxed)) {
+      }
     }
   }
   const int64_t col_tiles = (C + BC - 1) / BC;
