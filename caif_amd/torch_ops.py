@@ -225,3 +225,75 @@ def add(a, b):
 
 def silu_multiply(gate, up):
     return _ew("caifx_silu_multiply", 2, gate, up)
+
+
+# ------------------------------------------------------------------ MoE token routing
+def moe_build_dispatch_map(expert_indices, num_experts, capacity_per_expert=0):
+    """(dispatch_map [T, top_k] int32, expert_offsets [E+1] int32), built on the device without a host
+    round trip; expert_offsets[-1] is the number of assigned rows."""
+    _need_cuda(expert_indices)
+    assert expert_indices.dtype == torch.int32 and expert_indices.dim() == 2
+    T_, top_k = expert_indices.shape
+    dmap = torch.empty_like(expert_indices)
+    offsets = torch.empty(num_experts + 1, dtype=torch.int32, device=expert_indices.device)
+    nb = capi.lib().caifx_moe_dispatch_map_workspace_bytes(T_, top_k, num_experts)
+    ws = torch.empty(max(nb, 4 * num_experts), dtype=torch.uint8, device=expert_indices.device)
+    capi.call("caifx_moe_build_dispatch_map", _ptr(expert_indices), T_, top_k, num_experts, capacity_per_expert,
+              _ptr(dmap), _ptr(offsets), _ptr(ws), ws.numel(), _stream())
+    return dmap, offsets
+
+
+def moe_dispatch(x, expert_indices, dispatch_map, expert_offsets, total_rows, out=None):
+    _need_cuda(x, expert_indices, dispatch_map, expert_offsets)
+    T_, dim = x.shape
+    top_k = expert_indices.shape[1]
+    buf = out if out is not None else torch.zeros((total_rows, dim), dtype=x.dtype, device=x.device)
+    capi.call("caifx_moe_dispatch", _ptr(x), _ptr(expert_indices), _ptr(dispatch_map), _ptr(expert_offsets), _ptr(buf),
+              T_, dim, top_k, expert_offsets.numel() - 1, CODE_OF[x.dtype], _stream())
+    return buf
+
+
+def moe_combine(expert_buffer, expert_indices, expert_weights, dispatch_map, expert_offsets, out=None):
+    _need_cuda(expert_buffer, expert_indices, expert_weights, dispatch_map, expert_offsets)
+    T_, top_k = expert_indices.shape
+    dim = expert_buffer.shape[1]
+    y = out if out is not None else torch.empty((T_, dim), dtype=expert_buffer.dtype, device=expert_buffer.device)
+    capi.call("caifx_moe_combine", _ptr(expert_buffer), _ptr(expert_indices), _ptr(expert_weights), _ptr(dispatch_map),
+              _ptr(expert_offsets), _ptr(y), T_, dim, top_k, expert_offsets.numel() - 1, CODE_OF[expert_buffer.dtype],
+              _stream())
+    return y
+
+
+def moe_combine_backward_grad_expert(grad_output, expert_indices, expert_weights, dispatch_map, expert_offsets,
+                                     total_rows, out=None):
+    _need_cuda(grad_output, expert_indices, expert_weights, dispatch_map, expert_offsets)
+    T_, dim = grad_output.shape
+    top_k = expert_indices.shape[1]
+    gb = out if out is not None else torch.zeros((total_rows, dim), dtype=grad_output.dtype, device=grad_output.device)
+    capi.call("caifx_moe_combine_backward_grad_expert", _ptr(grad_output), _ptr(expert_indices), _ptr(expert_weights),
+              _ptr(dispatch_map), _ptr(expert_offsets), _ptr(gb), T_, dim, top_k, expert_offsets.numel() - 1,
+              CODE_OF[grad_output.dtype], _stream())
+    return gb
+
+
+def moe_dispatch_backward(grad_expert_buffer, expert_indices, dispatch_map, expert_offsets, out=None):
+    _need_cuda(grad_expert_buffer, expert_indices, dispatch_map, expert_offsets)
+    T_, top_k = expert_indices.shape
+    dim = grad_expert_buffer.shape[1]
+    gi = out if out is not None else torch.empty((T_, dim), dtype=grad_expert_buffer.dtype,
+                                                 device=grad_expert_buffer.device)
+    capi.call("caifx_moe_dispatch_backward", _ptr(grad_expert_buffer), _ptr(expert_indices), _ptr(dispatch_map),
+              _ptr(expert_offsets), _ptr(gi), T_, dim, top_k, expert_offsets.numel() - 1,
+              CODE_OF[grad_expert_buffer.dtype], _stream())
+    return gi
+
+
+def moe_combine_backward_grad_weights(grad_output, expert_buffer, expert_indices, dispatch_map, expert_offsets):
+    _need_cuda(grad_output, expert_buffer, expert_indices, dispatch_map, expert_offsets)
+    T_, top_k = expert_indices.shape
+    dim = grad_output.shape[1]
+    gw = torch.empty((T_, top_k), dtype=grad_output.dtype, device=grad_output.device)
+    capi.call("caifx_moe_combine_backward_grad_weights", _ptr(grad_output), _ptr(expert_buffer), _ptr(expert_indices),
+              _ptr(dispatch_map), _ptr(expert_offsets), _ptr(gw), T_, dim, top_k, expert_offsets.numel() - 1,
+              CODE_OF[grad_output.dtype], _stream())
+    return gw

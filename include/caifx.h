@@ -197,6 +197,70 @@ CAIFX_API int caifx_add(const void *a, const void *b, void *output, int64_t n, i
 CAIFX_API int caifx_silu_multiply(const void *gate, const void *up, void *hidden, int64_t n, int dtype,
                         caifx_stream_t stream);
 
+/* ---------------------------------------------------------------------------
+ * MoE token routing around the grouped dequant-GEMMs: the dispatch map, the gather into the
+ * token-sorted expert buffer, the weighted combine, and their backward passes.
+ * Shapes: expert_indices / dispatch_map / expert_weights [num_tokens, top_k] (indices and map
+ * int32, weights of `dtype`), expert_offsets int32 [num_experts + 1], token tensors
+ * [num_tokens, dim], expert buffer [offsets[num_experts], dim], all row-major on the device.
+ * An assignment whose expert index is outside [0, num_experts) or whose map entry is -1 (dropped
+ * by the capacity limit) moves no data, as in the reference kernels.
+ * ------------------------------------------------------------------------- */
+
+/* CAIF_Ops::MoEBuildDispatchMapDevice (src/caif_ops_device.cpp:4876-4960), which copies the indices
+ * to the host, loops there and copies map and offsets back.  Here everything stays on the device:
+ *   count_e = number of assignments (t,k) with index e; capacity_per_expert > 0 clamps it;
+ *   expert_offsets[e+1] = expert_offsets[e] + count_e;
+ *   dispatch_map[t,k] = number of assignments to the same expert that come earlier in token-major,
+ *   k-minor order, or -1 when that number is >= the clamped count (dropped).
+ * expert_offsets[num_experts] is the reference's return value (total assigned rows); callers that
+ * need it on the host read it back themselves.
+ * workspace: caifx_moe_dispatch_map_workspace_bytes(num_tokens, top_k, num_experts) bytes. */
+CAIFX_API size_t caifx_moe_dispatch_map_workspace_bytes(int64_t num_tokens, int top_k, int num_experts);
+CAIFX_API int caifx_moe_build_dispatch_map(const int32_t *expert_indices, int64_t num_tokens, int top_k, int num_experts,
+                                 int capacity_per_expert, int32_t *dispatch_map, int32_t *expert_offsets,
+                                 void *workspace, size_t workspace_bytes, caifx_stream_t stream);
+
+/* launch_moe_dispatch (include/caif/caif_cuda_kernels_moe.cuh:297-305, src/caif_cuda_kernels_moe.cu:616-647):
+ * expert_buffer[offsets[e(t,k)] + map[t,k]] = input[t]  (row copy, bit exact). */
+CAIFX_API int caifx_moe_dispatch(const void *input, const int32_t *expert_indices, const int32_t *dispatch_map,
+                       const int32_t *expert_offsets, void *expert_buffer, int64_t num_tokens, int64_t dim,
+                       int top_k, int num_experts, int dtype, caifx_stream_t stream);
+
+/* launch_moe_combine (caif_cuda_kernels_moe.cuh:317-326, caif_cuda_kernels_moe.cu:705-745):
+ * output[t,d] = T( sum over k in order of float(w[t,k]) * float(buffer[row(t,k), d]) ), fp32
+ * accumulation with one fused multiply-add per k, one rounding to T. */
+CAIFX_API int caifx_moe_combine(const void *expert_buffer, const int32_t *expert_indices, const void *expert_weights,
+                      const int32_t *dispatch_map, const int32_t *expert_offsets, void *output,
+                      int64_t num_tokens, int64_t dim, int top_k, int num_experts, int dtype,
+                      caifx_stream_t stream);
+
+/* launch_moe_combine_backward_grad_expert (caif_cuda_kernels_moe.cuh:333-342, caif_cuda_kernels_moe.cu:816-848):
+ * grad_expert_buffer[row(t,k), d] = T( float(w[t,k]) * float(grad_output[t,d]) ).  Rows no assignment
+ * maps to are left untouched, as in the reference. */
+CAIFX_API int caifx_moe_combine_backward_grad_expert(const void *grad_output, const int32_t *expert_indices,
+                                           const void *expert_weights, const int32_t *dispatch_map,
+                                           const int32_t *expert_offsets, void *grad_expert_buffer,
+                                           int64_t num_tokens, int64_t dim, int top_k, int num_experts, int dtype,
+                                           caifx_stream_t stream);
+
+/* launch_moe_combine_backward_grad_weights (caif_cuda_kernels_moe.cuh:349-358, caif_cuda_kernels_moe.cu:915-990):
+ * grad_weights[t,k] = T( sum over d of float(grad_output[t,d]) * float(buffer[row(t,k), d]) ), fp32
+ * accumulation; 0 for an assignment that moved no data.  The order of the additions is fixed but not the
+ * reference's block reduction, so parity is to fp32 rounding (1e-5 of the largest value), not bitwise. */
+CAIFX_API int caifx_moe_combine_backward_grad_weights(const void *grad_output, const void *expert_buffer,
+                                            const int32_t *expert_indices, const int32_t *dispatch_map,
+                                            const int32_t *expert_offsets, void *grad_weights,
+                                            int64_t num_tokens, int64_t dim, int top_k, int num_experts, int dtype,
+                                            caifx_stream_t stream);
+
+/* launch_moe_dispatch_backward (caif_cuda_kernels_moe.cuh:365-373, caif_cuda_kernels_moe.cu:1040-1071):
+ * grad_input[t,d] = T( sum over k in order of float(grad_expert_buffer[row(t,k), d]) ), fp32 sum. */
+CAIFX_API int caifx_moe_dispatch_backward(const void *grad_expert_buffer, const int32_t *expert_indices,
+                                const int32_t *dispatch_map, const int32_t *expert_offsets, void *grad_input,
+                                int64_t num_tokens, int64_t dim, int top_k, int num_experts, int dtype,
+                                caifx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -346,6 +346,98 @@ def moe_build_dispatch_map(indices, num_experts, capacity_per_expert=0):
     return dmap, offsets, int(total)
 
 
+def _routed_rows(indices, dmap, offsets, num_experts):
+    """Row of the expert buffer each assignment (t,k) maps to, -1 where it moves no data
+    (expert index out of range or map entry -1), as the reference kernels test it
+    (src/caif_cuda_kernels_moe.cu:640-645)."""
+    idx = np.asarray(indices, np.int64)
+    pos = np.asarray(dmap, np.int64)
+    ok = (idx >= 0) & (idx < num_experts) & (pos >= 0)
+    rows = np.where(ok, np.asarray(offsets, np.int64)[np.clip(idx, 0, num_experts - 1)] + pos, -1)
+    return rows
+
+
+def moe_dispatch(x_values, indices, dmap, offsets, num_experts, total_rows, dtype):
+    """moe_dispatch_kernel (src/caif_cuda_kernels_moe.cu:616-647): buffer[row(t,k)] = input[t]; rows no
+    assignment maps to keep their previous content (zeros here)."""
+    x = round_to_dtype(np.asarray(x_values, np.float32), dtype)
+    rows = _routed_rows(indices, dmap, offsets, num_experts)
+    buf = np.zeros((total_rows, x.shape[1]), np.float32)
+    T, top_k = rows.shape
+    for t in range(T):
+        for k in range(top_k):
+            if rows[t, k] >= 0:
+                buf[rows[t, k]] = x[t]
+    return buf
+
+
+def moe_combine(buffer_values, indices, weights, dmap, offsets, num_experts, dtype):
+    """moe_combine_kernel (src/caif_cuda_kernels_moe.cu:705-745): per (t,d) an fp32 sum over k in order,
+    sum += float(w) * float(buf) (one fused multiply-add, nvcc's default contraction), one rounding to T."""
+    buf = round_to_dtype(np.asarray(buffer_values, np.float32), dtype)
+    w = round_to_dtype(np.asarray(weights, np.float32), dtype)
+    rows = _routed_rows(indices, dmap, offsets, num_experts)
+    T, top_k = rows.shape
+    out = np.zeros((T, buf.shape[1]), np.float32)
+    for t in range(T):
+        acc = np.zeros(buf.shape[1], np.float64)        # exact product + one fp32 rounding per step = fmaf
+        acc32 = np.zeros(buf.shape[1], np.float32)
+        for k in range(top_k):
+            if rows[t, k] >= 0:
+                acc = np.float64(w[t, k]) * buf[rows[t, k]].astype(np.float64) + acc32.astype(np.float64)
+                acc32 = acc.astype(np.float32)
+        out[t] = acc32
+    return round_to_dtype(out, dtype)
+
+
+def moe_combine_backward_grad_expert(grad_values, indices, weights, dmap, offsets, num_experts, total_rows, dtype):
+    """moe_combine_backward_grad_expert_kernel (src/caif_cuda_kernels_moe.cu:816-848):
+    grad_buffer[row(t,k)] = T(float(w[t,k]) * float(grad_output[t])); other rows untouched (zeros here)."""
+    g = round_to_dtype(np.asarray(grad_values, np.float32), dtype)
+    w = round_to_dtype(np.asarray(weights, np.float32), dtype)
+    rows = _routed_rows(indices, dmap, offsets, num_experts)
+    out = np.zeros((total_rows, g.shape[1]), np.float32)
+    T, top_k = rows.shape
+    for t in range(T):
+        for k in range(top_k):
+            if rows[t, k] >= 0:
+                out[rows[t, k]] = round_to_dtype((w[t, k] * g[t]).astype(np.float32), dtype)
+    return out
+
+
+def moe_combine_backward_grad_weights(grad_values, buffer_values, indices, dmap, offsets, num_experts, dtype):
+    """moe_combine_backward_grad_weights_block_kernel (src/caif_cuda_kernels_moe.cu:915-990):
+    grad_weights[t,k] = T(sum_d float(grad_output[t,d]) * float(buffer[row(t,k),d])); 0 where the
+    assignment moved no data.  Accumulated in fp64 here (the reference's block-reduction order is not
+    part of its contract)."""
+    g = round_to_dtype(np.asarray(grad_values, np.float32), dtype).astype(np.float64)
+    buf = round_to_dtype(np.asarray(buffer_values, np.float32), dtype).astype(np.float64)
+    rows = _routed_rows(indices, dmap, offsets, num_experts)
+    T, top_k = rows.shape
+    out = np.zeros((T, top_k), np.float64)
+    for t in range(T):
+        for k in range(top_k):
+            if rows[t, k] >= 0:
+                out[t, k] = float(np.dot(g[t], buf[rows[t, k]]))
+    return round_to_dtype(out.astype(np.float32), dtype)
+
+
+def moe_dispatch_backward(grad_buffer_values, indices, dmap, offsets, num_experts, dtype):
+    """moe_dispatch_backward_kernel (src/caif_cuda_kernels_moe.cu:1040-1071): grad_input[t] =
+    T(sum over k in order of float(grad_buffer[row(t,k)])), fp32 additions."""
+    gb = round_to_dtype(np.asarray(grad_buffer_values, np.float32), dtype)
+    rows = _routed_rows(indices, dmap, offsets, num_experts)
+    T, top_k = rows.shape
+    out = np.zeros((T, gb.shape[1]), np.float32)
+    for t in range(T):
+        acc = np.zeros(gb.shape[1], np.float32)
+        for k in range(top_k):
+            if rows[t, k] >= 0:
+                acc = (acc + gb[rows[t, k]]).astype(np.float32)
+        out[t] = acc
+    return round_to_dtype(out, dtype)
+
+
 # --------------------------------------------------------------------------- LoRA around a frozen base
 def lora_forward(x_values, fw, lora_a, lora_b, alpha, compute_dtype, storage_dtype):
     """CAIF_DeviceLoRAAdapter::ForwardImpl (src/caif_device_lora_adapter.cpp:119-203):
