@@ -296,6 +296,28 @@ def moe_rows(torch, T, dev, gen):
         return e0.elapsed_time(e1) / iters
 
     ms_f, ms_b = timed(fwd), timed(bwd)
+    # token routing around the experts (dispatch map, gather, weighted combine, and their backward passes),
+    # on the same routing; HBM-bound row moves: algorithmic bytes = rows read + rows written
+    idx2 = ids.reshape(tokens, top_k).to(torch.int32).contiguous()
+    wts = torch.softmax(torch.empty(tokens, top_k, device=dev).normal_(0, 1, generator=gen), dim=1).to(torch.bfloat16)
+    xt = torch.empty(tokens, D, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16)
+    dmap, offs = T.moe_build_dispatch_map(idx2, E)
+    packed, comb, gbuf, gin = bf(rows, D), bf(tokens, D), bf(rows, D), bf(tokens, D)
+    row_b, tok_b = rows * D * 2, tokens * D * 2
+    routing = {}
+    for name, fn, nbytes in (
+            ("build_dispatch_map", lambda: T.moe_build_dispatch_map(idx2, E), None),
+            ("dispatch", lambda: T.moe_dispatch(xt, idx2, dmap, offs, rows, out=packed), tok_b + row_b),
+            ("combine", lambda: T.moe_combine(out, idx2, wts, dmap, offs, out=comb), row_b + tok_b),
+            ("combine_backward_grad_expert",
+             lambda: T.moe_combine_backward_grad_expert(comb, idx2, wts, dmap, offs, rows, out=gbuf), tok_b + row_b),
+            ("dispatch_backward", lambda: T.moe_dispatch_backward(gbuf, idx2, dmap, offs, out=gin), row_b + tok_b)):
+        ms = timed(fn, iters=20)
+        routing[name] = {"us": round(ms * 1e3, 2)}
+        if nbytes:
+            routing[name].update({"GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                  "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
+    routing_ms = sum(v["us"] for v in routing.values()) * 1e-3
     # per-expert-segment efficiency: replay single segments (shortest, median, longest) of the gate
     # projection as stand-alone dequant-GEMMs
     order = torch.argsort(counts).tolist()
@@ -312,6 +334,8 @@ def moe_rows(torch, T, dev, gen):
             "rows_per_expert_min_max": [int(counts.min()), int(counts.max())],
             "fwd_ms": round(ms_f, 4), "bwd_ms": round(ms_b, 4),
             "tokens_per_s_fwd_bwd": round(tokens / ((ms_f + ms_b) * 1e-3), 1),
+            "routing": routing,
+            "tokens_per_s_fwd_bwd_with_routing": round(tokens / ((ms_f + ms_b + routing_ms) * 1e-3), 1),
             "grouped_gemm_TFLOPs_fwd": round(gemm_flops / (ms_f * 1e-3) / 1e12, 1),
             "grouped_gemm_TFLOPs_bwd": round(gemm_flops / (ms_b * 1e-3) / 1e12, 1),
             "grouped_frac_of_mfma_peak": round(2 * gemm_flops / ((ms_f + ms_b) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),

@@ -54,20 +54,28 @@ __global__ __launch_bounds__(kRouteThreads) void map_count_kernel(const int32_t 
   }
 }
 
-// counts[w][e] -> exclusive prefix over w (in place); totals clamped by capacity -> offsets
-__global__ __launch_bounds__(kRouteThreads) void map_scan_kernel(int32_t *counts, int64_t slices, int num_experts,
-                                                                  int capacity, int32_t *offsets, int32_t *clamped)
+// counts[w][e] -> exclusive prefix over w (in place), one wave per expert walking the slices 64 at a
+// time; the total, clamped by the capacity, goes to clamped[e]
+__global__ __launch_bounds__(64) void map_scan_kernel(int32_t *counts, int64_t slices, int num_experts, int capacity,
+                                                       int32_t *clamped)
 {
-  const int e = blockIdx.x * kRouteThreads + threadIdx.x;
-  if (e >= num_experts) return;
-  int32_t run = 0;
-  for (int64_t w = 0; w < slices; ++w) {
-    const int32_t c = counts[w * num_experts + e];
-    counts[w * num_experts + e] = run;
-    run += c;
+  const int e = blockIdx.x;
+  const int lane = threadIdx.x;
+  int32_t carry = 0;
+  for (int64_t base = 0; base < slices; base += 64) {
+    const int64_t w = base + lane;
+    const int32_t c = w < slices ? counts[w * num_experts + e] : 0;
+    int32_t v = c;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int32_t up = __shfl_up(v, o, 64);
+      if (lane >= o) v += up;
+    }
+    if (w < slices) counts[w * num_experts + e] = carry + v - c;
+    carry += __shfl(v, 63, 64);
   }
-  if (capacity > 0 && run > capacity) run = capacity;
-  clamped[e] = run;
+  if (capacity > 0 && carry > capacity) carry = capacity;
+  if (lane == 0) clamped[e] = carry;
 }
 
 __global__ __launch_bounds__(64) void map_offsets_kernel(const int32_t *clamped, int num_experts, int32_t *offsets)
@@ -154,8 +162,8 @@ __global__ __launch_bounds__(kRouteThreads) void dispatch_kernel(const T *in, co
   }
 }
 
-// grad_expert_buffer[row(t,k)] = T(w[t,k] * grad_output[t])
-template <typename T>
+// grad_expert_buffer[row(t,k)] = T(w[t,k] * grad_output[t]); one wave per assignment
+template <typename T, bool kVec>
 __global__ __launch_bounds__(kRouteThreads) void combine_bwd_kernel(const T *gout, const int32_t *idx, const T *w,
                                                                      const int32_t *map, const int32_t *offsets, T *gbuf,
                                                                      int64_t assignments, int64_t dim, int top_k,
@@ -169,33 +177,77 @@ __global__ __launch_bounds__(kRouteThreads) void combine_bwd_kernel(const T *gou
   const float wt = to_f32<T>(w[a]);
   const T *src = gout + (a / top_k) * dim;
   T *dst = gbuf + row * dim;
-  for (int64_t d = lane; d < dim; d += 64) dst[d] = from_f32<T>(wt * to_f32<T>(src[d]));
+  if constexpr (kVec) {
+    typedef typename Vec16<T>::type v_t;
+    constexpr int n = Vec16<T>::kN;
+    for (int64_t d = lane * n; d < dim; d += 64 * n) {
+      const v_t g = *reinterpret_cast<const v_t *>(src + d);
+      v_t o;
+#pragma unroll
+      for (int i = 0; i < n; ++i) o[i] = from_f32<T>(wt * to_f32<T>(g[i]));
+      *reinterpret_cast<v_t *>(dst + d) = o;
+    }
+  } else {
+    for (int64_t d = lane; d < dim; d += 64) dst[d] = from_f32<T>(wt * to_f32<T>(src[d]));
+  }
 }
 
-// one wave per token: out[t] = T(sum_k w[t,k] * buf[row(t,k)])  (kWeighted) or T(sum_k buf[row(t,k)])
-template <typename T, bool kWeighted>
+// one wave per token: out[t] = T(sum_k w[t,k] * buf[row(t,k)])  (kWeighted) or T(sum_k buf[row(t,k)]);
+// per element the additions run over k in order.  The rows and weights of a token are fetched once per
+// batch of 8 assignments by lanes 0..7 and broadcast.
+template <typename T, bool kWeighted, bool kVec>
 __global__ __launch_bounds__(kRouteThreads) void gather_sum_kernel(const T *buf, const int32_t *idx, const T *w,
                                                                     const int32_t *map, const int32_t *offsets, T *out,
                                                                     int64_t num_tokens, int64_t dim, int top_k,
                                                                     int num_experts)
 {
+  constexpr int n = kVec ? Vec16<T>::kN : 1;
+  typedef typename Vec16<T>::type v_t;
   const int lane = threadIdx.x & 63;
   const int64_t t = (static_cast<int64_t>(blockIdx.x) * kRouteThreads + threadIdx.x) >> 6;
   if (t >= num_tokens) return;
-  for (int64_t d0 = 0; d0 < dim; d0 += 64) {
-    const int64_t d = d0 + lane;
-    float sum = 0.0f;
-    for (int k = 0; k < top_k; ++k) {
-      const int64_t a = t * top_k + k;
-      const int64_t row = routed_row(idx, map, offsets, a, num_experts);      // wave-uniform
-      if (row < 0) continue;
-      if (d < dim) {
-        const float v = to_f32<T>(buf[row * dim + d]);
-        if constexpr (kWeighted) sum = __builtin_fmaf(to_f32<T>(w[a]), v, sum);
-        else sum += v;
+  for (int64_t d0 = 0; d0 < dim; d0 += 64 * n) {          // the whole wave walks the row together
+    const int64_t d = d0 + static_cast<int64_t>(lane) * n;
+    float sum[n];
+#pragma unroll
+    for (int i = 0; i < n; ++i) sum[i] = 0.0f;
+    for (int k0 = 0; k0 < top_k; k0 += 8) {
+      int64_t my_row = -1;
+      float my_w = 0.0f;
+      if (lane < 8 && k0 + lane < top_k) {
+        const int64_t a = t * top_k + k0 + lane;
+        my_row = routed_row(idx, map, offsets, a, num_experts);
+        if constexpr (kWeighted) my_w = to_f32<T>(w[a]);
+      }
+      const int kn = top_k - k0 < 8 ? top_k - k0 : 8;
+      for (int k = 0; k < kn; ++k) {
+        const int64_t row = __shfl(my_row, k, 64);
+        const float wt = __shfl(my_w, k, 64);
+        if (row < 0 || d >= dim) continue;
+        if constexpr (kVec) {
+          const v_t v = *reinterpret_cast<const v_t *>(buf + row * dim + d);
+#pragma unroll
+          for (int i = 0; i < n; ++i) {
+            if constexpr (kWeighted) sum[i] = __builtin_fmaf(wt, to_f32<T>(v[i]), sum[i]);
+            else sum[i] += to_f32<T>(v[i]);
+          }
+        } else {
+          const float v = to_f32<T>(buf[row * dim + d]);
+          if constexpr (kWeighted) sum[0] = __builtin_fmaf(wt, v, sum[0]);
+          else sum[0] += v;
+        }
       }
     }
-    if (d < dim) out[t * dim + d] = from_f32<T>(sum);
+    if (d < dim) {
+      if constexpr (kVec) {
+        v_t o;
+#pragma unroll
+        for (int i = 0; i < n; ++i) o[i] = from_f32<T>(sum[i]);
+        *reinterpret_cast<v_t *>(out + t * dim + d) = o;
+      } else {
+        out[t * dim + d] = from_f32<T>(sum[0]);
+      }
+    }
   }
 }
 
@@ -271,8 +323,8 @@ int caifx_moe_build_dispatch_map(const int32_t *expert_indices, int64_t num_toke
   if (total > 0)
     hipLaunchKernelGGL(map_count_kernel, dim3(wave_blocks(slices)), dim3(kRouteThreads), 0, s, expert_indices, total,
                        num_experts, counts);
-  hipLaunchKernelGGL(map_scan_kernel, dim3((num_experts + kRouteThreads - 1) / kRouteThreads), dim3(kRouteThreads), 0, s,
-                     counts, slices, num_experts, capacity_per_expert, expert_offsets, clamped);
+  hipLaunchKernelGGL(map_scan_kernel, dim3(num_experts), dim3(64), 0, s, counts, slices, num_experts, capacity_per_expert,
+                     clamped);
   hipLaunchKernelGGL(map_offsets_kernel, dim3(1), dim3(64), 0, s, clamped, num_experts, expert_offsets);
   if (total > 0)
     hipLaunchKernelGGL(map_rank_kernel, dim3(wave_blocks(slices)), dim3(kRouteThreads), 0, s, expert_indices, total,
@@ -313,13 +365,23 @@ int caifx_moe_combine(const void *expert_buffer, const int32_t *expert_indices, 
   if (!expert_weights) return CAIFX_ERR_INVALID_ARGUMENT;
   const dim3 grid(wave_blocks(num_tokens)), block(kRouteThreads);
   hipStream_t s = as_stream(stream);
+  const bool vec = (dim * dtype_size(dtype)) % 16 == 0 && aligned_to(expert_buffer, 16) && aligned_to(output, 16);
 #define CAIFX_GO(T)                                                                                                    \
-  hipLaunchKernelGGL((gather_sum_kernel<T, true>), grid, block, 0, s, static_cast<const T *>(expert_buffer),           \
-                     expert_indices, static_cast<const T *>(expert_weights), dispatch_map, expert_offsets,            \
-                     static_cast<T *>(output), num_tokens, dim, top_k, num_experts)
-  if (dtype == CAIFX_F32) CAIFX_GO(float);
-  else if (dtype == CAIFX_F16) CAIFX_GO(f16_t);
-  else CAIFX_GO(bf16_t);
+  if (vec)                                                                                                             \
+    hipLaunchKernelGGL((gather_sum_kernel<T, true, true>), grid, block, 0, s, static_cast<const T *>(expert_buffer),   \
+                       expert_indices, static_cast<const T *>(expert_weights), dispatch_map, expert_offsets,          \
+                       static_cast<T *>(output), num_tokens, dim, top_k, num_experts);                                \
+  else                                                                                                                 \
+    hipLaunchKernelGGL((gather_sum_kernel<T, true, false>), grid, block, 0, s, static_cast<const T *>(expert_buffer),  \
+                       expert_indices, static_cast<const T *>(expert_weights), dispatch_map, expert_offsets,          \
+                       static_cast<T *>(output), num_tokens, dim, top_k, num_experts)
+  if (dtype == CAIFX_F32) {
+    CAIFX_GO(float);
+  } else if (dtype == CAIFX_F16) {
+    CAIFX_GO(f16_t);
+  } else {
+    CAIFX_GO(bf16_t);
+  }
 #undef CAIFX_GO
   return launch_status();
 }
@@ -336,13 +398,23 @@ int caifx_moe_combine_backward_grad_expert(const void *grad_output, const int32_
   const int64_t assignments = num_tokens * top_k;
   const dim3 grid(wave_blocks(assignments)), block(kRouteThreads);
   hipStream_t s = as_stream(stream);
+  const bool vec = (dim * dtype_size(dtype)) % 16 == 0 && aligned_to(grad_output, 16) && aligned_to(grad_expert_buffer, 16);
 #define CAIFX_GO(T)                                                                                                    \
-  hipLaunchKernelGGL(combine_bwd_kernel<T>, grid, block, 0, s, static_cast<const T *>(grad_output), expert_indices,    \
-                     static_cast<const T *>(expert_weights), dispatch_map, expert_offsets,                            \
-                     static_cast<T *>(grad_expert_buffer), assignments, dim, top_k, num_experts)
-  if (dtype == CAIFX_F32) CAIFX_GO(float);
-  else if (dtype == CAIFX_F16) CAIFX_GO(f16_t);
-  else CAIFX_GO(bf16_t);
+  if (vec)                                                                                                             \
+    hipLaunchKernelGGL((combine_bwd_kernel<T, true>), grid, block, 0, s, static_cast<const T *>(grad_output),          \
+                       expert_indices, static_cast<const T *>(expert_weights), dispatch_map, expert_offsets,          \
+                       static_cast<T *>(grad_expert_buffer), assignments, dim, top_k, num_experts);                   \
+  else                                                                                                                 \
+    hipLaunchKernelGGL((combine_bwd_kernel<T, false>), grid, block, 0, s, static_cast<const T *>(grad_output),         \
+                       expert_indices, static_cast<const T *>(expert_weights), dispatch_map, expert_offsets,          \
+                       static_cast<T *>(grad_expert_buffer), assignments, dim, top_k, num_experts)
+  if (dtype == CAIFX_F32) {
+    CAIFX_GO(float);
+  } else if (dtype == CAIFX_F16) {
+    CAIFX_GO(f16_t);
+  } else {
+    CAIFX_GO(bf16_t);
+  }
 #undef CAIFX_GO
   return launch_status();
 }
@@ -363,9 +435,13 @@ int caifx_moe_combine_backward_grad_weights(const void *grad_output, const void 
   hipLaunchKernelGGL(combine_bwd_weights_kernel<T>, grid, block, 0, s, static_cast<const T *>(grad_output),            \
                      static_cast<const T *>(expert_buffer), expert_indices, dispatch_map, expert_offsets,             \
                      static_cast<T *>(grad_weights), assignments, dim, top_k, num_experts)
-  if (dtype == CAIFX_F32) CAIFX_GO(float);
-  else if (dtype == CAIFX_F16) CAIFX_GO(f16_t);
-  else CAIFX_GO(bf16_t);
+  if (dtype == CAIFX_F32) {
+    CAIFX_GO(float);
+  } else if (dtype == CAIFX_F16) {
+    CAIFX_GO(f16_t);
+  } else {
+    CAIFX_GO(bf16_t);
+  }
 #undef CAIFX_GO
   return launch_status();
 }
@@ -379,13 +455,23 @@ int caifx_moe_dispatch_backward(const void *grad_expert_buffer, const int32_t *e
   if (st >= 0) return st;
   const dim3 grid(wave_blocks(num_tokens)), block(kRouteThreads);
   hipStream_t s = as_stream(stream);
+  const bool vec = (dim * dtype_size(dtype)) % 16 == 0 && aligned_to(grad_expert_buffer, 16) && aligned_to(grad_input, 16);
 #define CAIFX_GO(T)                                                                                                    \
-  hipLaunchKernelGGL((gather_sum_kernel<T, false>), grid, block, 0, s, static_cast<const T *>(grad_expert_buffer),     \
-                     expert_indices, static_cast<const T *>(nullptr), dispatch_map, expert_offsets,                   \
-                     static_cast<T *>(grad_input), num_tokens, dim, top_k, num_experts)
-  if (dtype == CAIFX_F32) CAIFX_GO(float);
-  else if (dtype == CAIFX_F16) CAIFX_GO(f16_t);
-  else CAIFX_GO(bf16_t);
+  if (vec)                                                                                                             \
+    hipLaunchKernelGGL((gather_sum_kernel<T, false, true>), grid, block, 0, s,                                         \
+                       static_cast<const T *>(grad_expert_buffer), expert_indices, static_cast<const T *>(nullptr),   \
+                       dispatch_map, expert_offsets, static_cast<T *>(grad_input), num_tokens, dim, top_k, num_experts); \
+  else                                                                                                                 \
+    hipLaunchKernelGGL((gather_sum_kernel<T, false, false>), grid, block, 0, s,                                        \
+                       static_cast<const T *>(grad_expert_buffer), expert_indices, static_cast<const T *>(nullptr),   \
+                       dispatch_map, expert_offsets, static_cast<T *>(grad_input), num_tokens, dim, top_k, num_experts)
+  if (dtype == CAIFX_F32) {
+    CAIFX_GO(float);
+  } else if (dtype == CAIFX_F16) {
+    CAIFX_GO(f16_t);
+  } else {
+    CAIFX_GO(bf16_t);
+  }
 #undef CAIFX_GO
   return launch_status();
 }
