@@ -4,8 +4,10 @@
 // call lands in one C-ABI launcher of caifx.h; a non-zero status becomes a CAIF_Exception.
 #pragma once
 
+#include <algorithm>
 #include <cstdint>
 #include <string>
+#include <vector>
 
 #include "caif_device_tensor.h"
 #include "caif_run_context.h"
@@ -210,6 +212,120 @@ class CAIF_Ops
       CAIF_CATCH_BLOCK()
     }
 
+    // ---- MoE token routing (include/caif/caif_ops.h:1234-1326 of the reference) ----------------------
+    // expert_indices and dispatch_map hold int32 [num_tokens, top_k], expert_offsets int32 [num_experts+1].
+
+    // Returns the number of assigned rows like the reference (src/caif_ops_device.cpp:4876-4960), which makes
+    // this call synchronise the stream for one 4-byte copy; map and offsets themselves never leave the device.
+    static uint32_t MoEBuildDispatchMap(const CAIF_DeviceTensor &expert_indices,uint32_t num_experts,uint32_t top_k,
+                                        uint32_t capacity_per_expert,CAIF_DeviceTensor &dispatch_map,
+                                        CAIF_DeviceTensor &expert_offsets)
+    {
+      try
+      {
+        RequireDevice(expert_indices,"MoEBuildDispatchMap");
+        if(expert_indices.Shape().size()!=2)
+        {
+          THROW_CAIFE("MoEBuildDispatchMap: expert_indices must be 2D [num_tokens x top_k]");
+        }
+        if(!FourByte(expert_indices)||!FourByte(dispatch_map)||!FourByte(expert_offsets))
+        {
+          THROW_CAIFE("MoEBuildDispatchMap: indices, map and offsets must hold 32-bit integers");
+        }
+        const uint32_t num_tokens=expert_indices.Shape()[0];
+        if(expert_indices.Shape()[1]!=top_k||dispatch_map.TotalElements()!=expert_indices.TotalElements()||
+           expert_offsets.TotalElements()!=static_cast<size_t>(num_experts)+1)
+        {
+          THROW_CAIFE("MoEBuildDispatchMap: shape mismatch");
+        }
+        const size_t ws_bytes=std::max<size_t>(caifx_moe_dispatch_map_workspace_bytes(num_tokens,static_cast<int>(top_k),
+                                                                                      static_cast<int>(num_experts)),
+                                               static_cast<size_t>(num_experts)*4);
+        CAIF_DeviceTensor ws=CAIF_DeviceTensor::Uninitialized({static_cast<uint32_t>(ws_bytes)},
+                                                              CAIF_CudaStream::Wrap(expert_offsets.StreamHandle()),
+                                                              Dtype_e::UInt8);
+        Check(caifx_moe_build_dispatch_map(static_cast<const int32_t*>(expert_indices.DeviceDataRaw()),num_tokens,
+                                           static_cast<int>(top_k),static_cast<int>(num_experts),
+                                           static_cast<int>(capacity_per_expert),
+                                           static_cast<int32_t*>(dispatch_map.DeviceDataRaw()),
+                                           static_cast<int32_t*>(expert_offsets.DeviceDataRaw()),ws.DeviceDataRaw(),ws_bytes,
+                                           expert_offsets.StreamHandle()),"MoEBuildDispatchMap");
+        std::vector<int32_t> offsets(static_cast<size_t>(num_experts)+1);
+        expert_offsets.CopyToHostRaw(offsets.data());
+        return static_cast<uint32_t>(offsets[num_experts]);
+      }
+      CAIF_CATCH_BLOCK()
+    }
+    static void MoEDispatchGPU(const CAIF_DeviceTensor &input,const CAIF_DeviceTensor &expert_indices,
+                               const CAIF_DeviceTensor &dispatch_map,const CAIF_DeviceTensor &expert_offsets,uint32_t top_k,
+                               CAIF_DeviceTensor &expert_buffer)
+    {
+      try
+      {
+        RouteShapes(input,expert_indices,dispatch_map,expert_offsets,top_k,expert_buffer,"MoEDispatchGPU");
+        Check(caifx_moe_dispatch(input.DeviceDataRaw(),Idx(expert_indices),Idx(dispatch_map),Idx(expert_offsets),
+                                 expert_buffer.DeviceDataRaw(),input.Shape()[0],input.Shape()[1],static_cast<int>(top_k),
+                                 Experts(expert_offsets),CAIF_DataType(input.Dtype()).CaifxCode(),expert_buffer.StreamHandle()),
+              "MoEDispatchGPU");
+      }
+      CAIF_CATCH_BLOCK()
+    }
+    static void MoECombineGPU(const CAIF_DeviceTensor &expert_buffer,const CAIF_DeviceTensor &expert_indices,
+                              const CAIF_DeviceTensor &expert_weights,const CAIF_DeviceTensor &dispatch_map,
+                              const CAIF_DeviceTensor &expert_offsets,uint32_t top_k,CAIF_DeviceTensor &output)
+    {
+      try
+      {
+        RouteShapes(output,expert_indices,dispatch_map,expert_offsets,top_k,expert_buffer,"MoECombineGPU");
+        RouteWeights(expert_weights,expert_indices,output,"MoECombineGPU");
+        Check(caifx_moe_combine(expert_buffer.DeviceDataRaw(),Idx(expert_indices),expert_weights.DeviceDataRaw(),
+                                Idx(dispatch_map),Idx(expert_offsets),output.DeviceDataRaw(),output.Shape()[0],
+                                output.Shape()[1],static_cast<int>(top_k),Experts(expert_offsets),
+                                CAIF_DataType(output.Dtype()).CaifxCode(),output.StreamHandle()),"MoECombineGPU");
+      }
+      CAIF_CATCH_BLOCK()
+    }
+    static void MoECombineBackwardGPU(const CAIF_DeviceTensor &grad_output,const CAIF_DeviceTensor &expert_buffer,
+                                      const CAIF_DeviceTensor &expert_indices,const CAIF_DeviceTensor &expert_weights,
+                                      const CAIF_DeviceTensor &dispatch_map,const CAIF_DeviceTensor &expert_offsets,
+                                      uint32_t top_k,CAIF_DeviceTensor &grad_expert_buffer,CAIF_DeviceTensor &grad_weights)
+    {
+      try
+      {
+        RouteShapes(grad_output,expert_indices,dispatch_map,expert_offsets,top_k,grad_expert_buffer,"MoECombineBackwardGPU");
+        RouteWeights(expert_weights,expert_indices,grad_output,"MoECombineBackwardGPU");
+        RouteWeights(grad_weights,expert_indices,grad_output,"MoECombineBackwardGPU");
+        SameKind(expert_buffer,grad_expert_buffer,"MoECombineBackwardGPU");
+        const int code=CAIF_DataType(grad_output.Dtype()).CaifxCode();
+        Check(caifx_moe_combine_backward_grad_expert(grad_output.DeviceDataRaw(),Idx(expert_indices),
+                                                     expert_weights.DeviceDataRaw(),Idx(dispatch_map),Idx(expert_offsets),
+                                                     grad_expert_buffer.DeviceDataRaw(),grad_output.Shape()[0],
+                                                     grad_output.Shape()[1],static_cast<int>(top_k),Experts(expert_offsets),
+                                                     code,grad_expert_buffer.StreamHandle()),"MoECombineBackwardGPU");
+        Check(caifx_moe_combine_backward_grad_weights(grad_output.DeviceDataRaw(),expert_buffer.DeviceDataRaw(),
+                                                      Idx(expert_indices),Idx(dispatch_map),Idx(expert_offsets),
+                                                      grad_weights.DeviceDataRaw(),grad_output.Shape()[0],
+                                                      grad_output.Shape()[1],static_cast<int>(top_k),Experts(expert_offsets),
+                                                      code,grad_weights.StreamHandle()),"MoECombineBackwardGPU");
+      }
+      CAIF_CATCH_BLOCK()
+    }
+    static void MoEDispatchBackwardGPU(const CAIF_DeviceTensor &grad_expert_buffer,const CAIF_DeviceTensor &expert_indices,
+                                       const CAIF_DeviceTensor &dispatch_map,const CAIF_DeviceTensor &expert_offsets,
+                                       uint32_t top_k,CAIF_DeviceTensor &grad_input)
+    {
+      try
+      {
+        RouteShapes(grad_input,expert_indices,dispatch_map,expert_offsets,top_k,grad_expert_buffer,"MoEDispatchBackwardGPU");
+        Check(caifx_moe_dispatch_backward(grad_expert_buffer.DeviceDataRaw(),Idx(expert_indices),Idx(dispatch_map),
+                                          Idx(expert_offsets),grad_input.DeviceDataRaw(),grad_input.Shape()[0],
+                                          grad_input.Shape()[1],static_cast<int>(top_k),Experts(expert_offsets),
+                                          CAIF_DataType(grad_input.Dtype()).CaifxCode(),grad_input.StreamHandle()),
+              "MoEDispatchBackwardGPU");
+      }
+      CAIF_CATCH_BLOCK()
+    }
+
     // Map a C-ABI status to the reference's error convention.
     static void Check(int status,const char *what)
     {
@@ -220,6 +336,39 @@ class CAIF_Ops
     }
 
   private:
+    // The reference keeps these int32 arrays in tensors of its default dtype (Float32): only the
+    // element size is part of the contract (tests/test_device_moe.cpp:1574-1583).
+    static bool FourByte(const CAIF_DeviceTensor &t){return t.Dtype()==Dtype_e::Int32||t.Dtype()==Dtype_e::Float32;}
+    static const int32_t *Idx(const CAIF_DeviceTensor &t){return static_cast<const int32_t*>(t.DeviceDataRaw());}
+    static int Experts(const CAIF_DeviceTensor &offsets){return static_cast<int>(offsets.TotalElements())-1;}
+    // tokens [T, dim] and buffer [rows, dim] of one float dtype; indices / map Int32 [T, top_k]; offsets Int32
+    static void RouteShapes(const CAIF_DeviceTensor &tokens,const CAIF_DeviceTensor &indices,const CAIF_DeviceTensor &map,
+                            const CAIF_DeviceTensor &offsets,uint32_t top_k,const CAIF_DeviceTensor &buffer,const char *op)
+    {
+      RequireDevice(tokens,op);
+      RequireDevice(buffer,op);
+      if(tokens.Shape().size()!=2||buffer.Shape().size()!=2||indices.Shape().size()!=2)
+      {
+        THROW_CAIFE(std::string(op)+": tokens, buffer and indices must be 2D");
+      }
+      if(!FourByte(indices)||!FourByte(map)||!FourByte(offsets))
+      {
+        THROW_CAIFE(std::string(op)+": indices, map and offsets must hold 32-bit integers");
+      }
+      if(tokens.Dtype()!=buffer.Dtype()||tokens.Shape()[1]!=buffer.Shape()[1]||indices.Shape()[0]!=tokens.Shape()[0]||
+         indices.Shape()[1]!=top_k||map.TotalElements()!=indices.TotalElements()||offsets.TotalElements()<2)
+      {
+        THROW_CAIFE(std::string(op)+": shape or dtype mismatch");
+      }
+    }
+    static void RouteWeights(const CAIF_DeviceTensor &weights,const CAIF_DeviceTensor &indices,const CAIF_DeviceTensor &like,
+                             const char *op)
+    {
+      if(weights.Dtype()!=like.Dtype()||weights.TotalElements()!=indices.TotalElements())
+      {
+        THROW_CAIFE(std::string(op)+": routing weights must be [num_tokens x top_k] of the token dtype");
+      }
+    }
     static void RequireDevice(const CAIF_DeviceTensor &t,const char *op)
     {
       if(t.Location()==CAIF_DeviceTensor::Location_e::Host_e)

@@ -9,7 +9,7 @@ import subprocess
 import pytest
 
 BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "bin")
-PROGRAMS = ["test_quantize_ops", "test_device_frozen_linear", "test_device_moe_frozen_expert"]
+PROGRAMS = ["test_quantize_ops", "test_device_frozen_linear", "test_device_moe_frozen_expert", "test_moe_routing"]
 
 
 def _run(name, args):
