@@ -99,18 +99,36 @@ __device__ __forceinline__ void store_out(void *y, int y_dtype, int64_t o, float
   else static_cast<f16_t *>(y)[o] = from_f32<f16_t>(v);
 }
 
+// (a & mask) | base in one instruction (the compiler splits it in two when both constants are literals)
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t base)
+{
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(base));
+  return r;
+}
+
+constexpr int kSegBlocks = 16;                         // row blocks between two flushes of the output staging buffer
+constexpr int kSegRows = kSegBlocks * 16;
+
 // GPW: 128-k groups per wave (K <= 16 * GPW * 128); 1 and 2 fit the 128 registers of a 1024-thread workgroup
+//
+// Memory requests are arranged so that the compiler can count them: the weight loads are never
+// behind a branch (lanes past the last row re-read the last row, row blocks past the end read the
+// first bytes of the weight) and no global store happens between them (results are staged in LDS
+// and written once per kSegRows rows).  A wait for one block of the ring then leaves the younger
+// block in flight instead of draining the queue.
 template <typename CT, typename XT, bool kInt4, int GPW>
 __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
 {
   typedef typename Mfma16<CT>::vec_t vec_t;
   constexpr int LPG = kInt4 ? 1 : 2;           // 16-byte loads per lane per 128-k group
   constexpr int LPR = GPW * LPG;               // ... per block of 16 weight rows
-  constexpr int D = LPR >= 4 ? 1 : 4 / LPR;    // row blocks in flight (4 loads per lane)
-  constexpr int RBB = kInt4 ? 4 : 2;           // row blocks between two reductions (a multiple of D)
+  constexpr int D = 2;                         // row blocks in the ring
+  constexpr int RBB = kInt4 ? 4 : 2;           // row blocks between two reductions (a multiple of D, divides kSegBlocks)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float *partial = reinterpret_cast<float *>(smem);      // [RBB][16 waves][4][64]
-  float *svec = partial + RBB * kPartialFloats;          // int8 with a scale vector: [K]
+  float *ybuf = partial + RBB * kPartialFloats;          // [16 activation rows][kSegRows]
+  float *svec = ybuf + 16 * kSegRows;                    // int8 with a scale vector: [K]
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -125,6 +143,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
   const int64_t i_lo = bc * per_block;
   const int64_t i_hi = i_lo + per_block < rows_class ? i_lo + per_block : rows_class;
   const int nrb = i_hi > i_lo ? static_cast<int>((i_hi - i_lo + 15) / 16) : 0;
+  if (nrb == 0) return;           // the whole workgroup; nothing has been started yet
   const int g0 = wave * GPW;
   const f16_t *s16 = static_cast<const f16_t *>(a.scales);
   const float *s32 = static_cast<const float *>(a.scales);
@@ -132,63 +151,75 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
   u32x4_t w[D][LPR];
   f16_t sc[D][GPW];
   auto issue = [&](int d, int rb) {
-    const int64_t i = i_lo + static_cast<int64_t>(rb) * 16 + j;
-    if (i < i_hi) {                    // masked lanes fetch nothing; their columns of the tile are never stored
-      const int64_t f0 = (cls + a.V * i) * a.K;
+    int64_t i = i_lo + static_cast<int64_t>(rb) * 16 + j;
+    if (i >= i_hi) i = i_hi - 1;                                   // masked lanes: their columns of the tile are never stored
+    const int64_t f0 = rb < nrb ? (cls + a.V * i) * a.K : 0;       // (wave uniform) past the end: the first weight row
 #pragma unroll
-      for (int g = 0; g < GPW; ++g) {
-        const int gg = g0 + g;
-        if (gg < a.groups) {
-          const int64_t f = f0 + gg * 128;
-          if constexpr (kInt4) {
-            w[d][g] = *reinterpret_cast<const u32x4_t *>(a.wq + (f >> 1) + q * 16);
-            sc[d][g] = s16[f >> a.group_shift];
-          } else {
-            w[d][2 * g] = *reinterpret_cast<const u32x4_t *>(a.wq + f + q * 16);
-            w[d][2 * g + 1] = *reinterpret_cast<const u32x4_t *>(a.wq + f + 64 + q * 16);
-          }
-        }
+    for (int g = 0; g < GPW; ++g) {
+      const int gg = g0 + g < a.groups ? g0 + g : a.groups - 1;   // waves without a k range compute on zero activations
+      const int64_t f = f0 + gg * 128;
+      if constexpr (kInt4) {
+        w[d][g] = *reinterpret_cast<const u32x4_t *>(a.wq + (f >> 1) + q * 16);
+        sc[d][g] = s16[f >> a.group_shift];
+      } else {
+        w[d][2 * g] = *reinterpret_cast<const u32x4_t *>(a.wq + f + q * 16);
+        w[d][2 * g + 1] = *reinterpret_cast<const u32x4_t *>(a.wq + f + 64 + q * 16);
       }
     }
   };
-  // Order of the requests: this wave's slice of X first (it comes from L2 and is needed first),
-  // then the first weight blocks; loads return in order, so X can be turned into A operands while
-  // the weights are still on their way from HBM.
+  // Order of the requests: this wave's slice of X and (int8) the scale vector first, they come from
+  // L2 and are needed first; then the first weight blocks.  Loads return in order, so the prologue
+  // runs while the weights are still on their way from HBM.
   vec_t xa[GPW][4];
   {
-    const XT *xg = static_cast<const XT *>(a.x) + static_cast<int64_t>(j < a.M ? j : 0) * a.K;
+    const XT *xg = static_cast<const XT *>(a.x) + static_cast<int64_t>(j < a.M ? j : a.M - 1) * a.K;
 #pragma unroll
     for (int g = 0; g < GPW; ++g) {
-      const int gg = g0 + g;
+      const int gg = g0 + g < a.groups ? g0 + g : a.groups - 1;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        vec_t v;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = from_f32<CT>(0.0f);
-        if (gg < a.groups && j < a.M) {
-          const int k = kInt4 ? gg * 128 + q * 32 + 8 * t : gg * 128 + (t >> 1) * 64 + q * 16 + 8 * (t & 1);
-          v = load_x8<CT, XT>(xg + k);
-        }
-        xa[g][t] = v;
+        const int k = kInt4 ? gg * 128 + q * 32 + 8 * t : gg * 128 + (t >> 1) * 64 + q * 16 + 8 * (t & 1);
+        xa[g][t] = load_x8<CT, XT>(xg + k);
       }
     }
   }
-#pragma unroll
-  for (int d = 0; d < D; ++d)
-    if (d < nrb) issue(d, d);
-
-  // int8 scale vector of this residue class: svec[k] = scales[(cls*K + k) mod period]
+  // int8 scale vector of this residue class: svec[k] = scales[(cls*K + k) mod period], K <= 4096
   float s_one = 1.0f;
+  float sv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   if constexpr (!kInt4) {
     if (a.period > 0) {
       int idx = static_cast<int>((static_cast<int64_t>(cls) * a.K + threadIdx.x) % a.period);
-      for (int64_t k = threadIdx.x; k < a.K; k += kMbThreads) {
-        svec[k] = s32[idx];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        sv[t] = s32[idx];
         idx += a.scale_step;
         if (idx >= a.period) idx -= a.period;
       }
     } else if (a.scales) {
       s_one = s32[0];
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < D; ++d) issue(d, d);
+
+  {
+    vec_t zero;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) zero[i] = from_f32<CT>(0.0f);
+#pragma unroll
+    for (int g = 0; g < GPW; ++g) {
+      const bool live = g0 + g < a.groups && j < a.M;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) xa[g][t] = live ? xa[g][t] : zero;
+    }
+  }
+  if constexpr (!kInt4) {
+    if (a.period > 0) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int k = threadIdx.x + t * kMbThreads;
+        if (k < a.K) svec[k] = sv[t];
+      }
     }
   }
 
@@ -223,48 +254,44 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
 
   // The waves run freely through RBB blocks of 16 rows (no barrier in between, so one wave's
   // arithmetic overlaps another's wait for HBM), then the 16 partial tiles of each block are added
-  // through LDS in a fixed order.
-  for (int base = 0; base < nrb; base += RBB) {
-    floatx4_t tot[RBB];
+  // through LDS in a fixed order into the staging buffer.
+  for (int seg0 = 0; seg0 < nrb; seg0 += kSegBlocks) {
+    const int seg_end = seg0 + kSegBlocks < nrb ? seg0 + kSegBlocks : nrb;
+    for (int base = seg0; base < seg_end; base += RBB) {
+      floatx4_t tot[RBB];
 #pragma unroll
-    for (int u = 0; u < RBB; ++u) {
-      const int d = u % D;
-      const int rb = base + u;
-      tot[u] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
-      if (rb < nrb) {          // same for every thread of the workgroup
-        u32x4_t wr[LPR];
-        float sr[GPW];
+      for (int u = 0; u < RBB; ++u) {
+        const int d = u % D;
+        const int rb = base + u;
+        tot[u] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        if (rb < nrb) {          // same for every thread of the workgroup
 #pragma unroll
-        for (int i = 0; i < LPR; ++i) wr[i] = w[d][i];
-        if constexpr (kInt4) {
-#pragma unroll
-          for (int g = 0; g < GPW; ++g) sr[g] = to_f32(sc[d][g]);
-        }
-        if (rb + D < nrb) issue(d, rb + D);
-#pragma unroll
-        for (int g = 0; g < GPW; ++g) {
-          const int gg = g0 + g;
-          if (gg < a.groups) {
+          for (int g = 0; g < GPW; ++g) {
             if constexpr (kInt4) {
               floatx4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
               for (int t = 0; t < 4; ++t) {
-                const uint32_t p = wr[g][t];
+                // one xor turns the eight two's-complement nibbles into code + 8; every pair of
+                // nibbles then takes a shift and one and-or to become OFFSET-biased values
+                const uint32_t p = w[d][g][t] ^ 0x88888888u;
+                constexpr uint32_t kBase = Mfma16<CT>::kMagic & 0xFFF0FFF0u;
                 u32x4_t c4;
-                c4[0] = (p & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
-                c4[1] = ((p >> 4) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
-                c4[2] = ((p >> 8) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
-                c4[3] = ((p >> 12) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
+                c4[0] = and_or(p, 0x000F000Fu, kBase);
+                c4[1] = and_or(p >> 4, 0x000F000Fu, kBase);
+                c4[2] = and_or(p >> 8, 0x000F000Fu, kBase);
+                c4[3] = and_or(p >> 12, 0x000F000Fu, kBase);
                 acc = Mfma16<CT>::run(xa[g][t], *reinterpret_cast<const vec_t *>(&c4), acc);
               }
+              const float sr = to_f32(sc[d][g]);
 #pragma unroll
-              for (int r = 0; r < 4; ++r) tot[u][r] = __builtin_fmaf(sr[g], acc[r] - cor[g][r], tot[u][r]);
+              for (int r = 0; r < 4; ++r) tot[u][r] = __builtin_fmaf(sr, acc[r] - cor[g][r], tot[u][r]);
             } else {
+              const int gg = g0 + g < a.groups ? g0 + g : a.groups - 1;
 #pragma unroll
               for (int t = 0; t < 4; ++t) {
                 float lo[4], hi[4];
-                int8x4_to_f32(wr[2 * g + (t >> 1)][2 * (t & 1)], lo);
-                int8x4_to_f32(wr[2 * g + (t >> 1)][2 * (t & 1) + 1], hi);
+                int8x4_to_f32(w[d][2 * g + (t >> 1)][2 * (t & 1)], lo);
+                int8x4_to_f32(w[d][2 * g + (t >> 1)][2 * (t & 1) + 1], hi);
                 floatx4_t s0 = {s_one, s_one, s_one, s_one};
                 floatx4_t s1 = s0;
                 if (a.period > 0) {
@@ -283,27 +310,35 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
             }
           }
         }
+        issue(d, rb + D);      // into the registers just consumed; the other block of the ring stays in flight
       }
-    }
 
-    // tot[u][r] = this wave's share of Y[activation row 4q+r][weight row j of block base+u]
+      // tot[u][r] = this wave's share of Y[activation row 4q+r][weight row j of block base+u]
 #pragma unroll
-    for (int u = 0; u < RBB; ++u)
+      for (int u = 0; u < RBB; ++u)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) partial[((u * kMbWaves + wave) * 4 + r) * 64 + lane] = tot[u][r];
-    __syncthreads();
-    if (threadIdx.x < RBB * 256) {
-      const int u = threadIdx.x >> 8;
-      const int r = (threadIdx.x >> 6) & 3;
-      const int l = threadIdx.x & 63;
-      float v = 0.0f;
+        for (int r = 0; r < 4; ++r) partial[((u * kMbWaves + wave) * 4 + r) * 64 + lane] = tot[u][r];
+      __syncthreads();
+      if (threadIdx.x < RBB * 256) {
+        const int u = threadIdx.x >> 8;
+        const int r = (threadIdx.x >> 6) & 3;
+        const int l = threadIdx.x & 63;
+        float v = 0.0f;
 #pragma unroll
-      for (int wv = 0; wv < kMbWaves; ++wv) v += partial[((u * kMbWaves + wv) * 4 + r) * 64 + l];
-      const int m = 4 * (l >> 4) + r;
-      const int64_t i = i_lo + static_cast<int64_t>(base + u) * 16 + (l & 15);
-      if (m < a.M && i < i_hi) store_out(a.y, a.y_dtype, static_cast<int64_t>(m) * a.N + cls + a.V * i, v);
+        for (int wv = 0; wv < kMbWaves; ++wv) v += partial[((u * kMbWaves + wv) * 4 + r) * 64 + l];
+        const int m = 4 * (l >> 4) + r;
+        ybuf[m * kSegRows + (base - seg0 + u) * 16 + (l & 15)] = v;
+      }
+      __syncthreads();            // the next round overwrites the partial tiles; the flush reads ybuf
     }
-    if (base + RBB < nrb) __syncthreads();      // the next round overwrites the partial tiles
+    // flush: Y[m][cls + V*i] for the rows of this segment
+    const int64_t i_seg = i_lo + static_cast<int64_t>(seg0) * 16;
+    const int seg_rows = static_cast<int>(i_hi - i_seg < kSegRows ? i_hi - i_seg : kSegRows);
+    for (int idx = threadIdx.x; idx < a.M * seg_rows; idx += kMbThreads) {
+      const int m = idx / seg_rows;
+      const int r = idx - m * seg_rows;
+      store_out(a.y, a.y_dtype, static_cast<int64_t>(m) * a.N + cls + a.V * (i_seg + r), ybuf[m * kSegRows + r]);
+    }
   }
 }
 
@@ -369,7 +404,7 @@ int mblock_forward(const GemmArgs &g, hipStream_t s)
   m.K = g.K;
   m.groups = static_cast<int>(g.K / 128);
   m.V = 1;
-  size_t lds = (int4 ? 4 : 2) * kPartialFloats * sizeof(float);      // RBB buffers of partial tiles
+  size_t lds = ((int4 ? 4 : 2) * kPartialFloats + 16 * kSegRows) * sizeof(float);      // RBB buffers of partial tiles + output staging
   if (int4) {
     const int gs = g.w.group_size;
     if (!g.w.scales || gs < 128 || (gs & (gs - 1)) != 0) return CAIFX_ERR_UNSUPPORTED;

@@ -4,7 +4,7 @@
 // K=4096 x N=14336 case takes about 6 us, and any pattern that touches 64-byte pieces of 16
 // different rows per instruction is 20-50 % slower than that.  Here one load instruction of a
 // wave covers 1 KiB of ONE weight row (lane l reads bytes [16 l, 16 l + 16)), a wave walks a
-// few whole rows, and a lane keeps 8 such loads in flight.
+// few whole rows through a small ring of rows in flight.
 //
 // The matrix core still does the multiply-adds.  v_mfma_f32_16x16x32 wants, per lane
 // (i = lane%16, c = lane/16), 8 consecutive-k values of "row i" of A and of "column i" of B.
@@ -118,6 +118,21 @@ __device__ __forceinline__ float wave_sum_hi(float v)
   v = dpp_add<0x142, 0xA>(v);   // row_bcast:15 into rows 1 and 3
   v = dpp_add<0x143, 0xC>(v);   // row_bcast:31 into rows 2 and 3
   return v;
+}
+
+// (a & mask) | base in one instruction (the compiler splits it in two when both constants are literals)
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t base)
+{
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(base));
+  return r;
+}
+
+// `acc` with lane `dst_lane` (wave uniform) replaced by the wave sum that wave_sum_hi left in lane 63
+__device__ __forceinline__ float lane_insert(float acc, float sum_hi, int dst_lane)
+{
+  const int s = __builtin_amdgcn_readlane(__builtin_bit_cast(int, sum_hi), 63);
+  return static_cast<int>(threadIdx.x & 63) == dst_lane ? __builtin_bit_cast(float, s) : acc;
 }
 
 __device__ __forceinline__ void store_y(void *y, int y_dtype, int64_t o, float v)
@@ -295,10 +310,14 @@ __global__ __launch_bounds__(256) void rowlin_int4_kernel(RowArgs a)
 
 // ------------------------------------------------------------------ fixed-shape fast paths
 // Same arithmetic as the kernels above for rows made of whole chunks (K = CPR * 2048 for int4,
-// CPR * 1024 for int8).  Every inner trip count is a compile-time constant; the activations are
-// requested BEFORE the first weight loads so that staging them does not wait for the weights
-// (loads return in order); a wave walks `rows_per_wave` rows through a ring of 8/CPR rows in
-// flight, so unpacking one row overlaps the HBM latency of the next ones.
+// CPR * 1024 for int8).  Every inner trip count is a compile-time constant.  What the prologue needs
+// (activations, int8 scales) is requested BEFORE the first weight rows, because loads return in
+// order; a wave then walks `rows_per_wave` rows through a ring of D rows: it computes a row out of
+// the registers it arrived in and requests the row D further on into the same registers, so D-1
+// rows are on their way from HBM while one is unpacked.  No load sits behind a branch (rows past the
+// end read a cache-resident dummy) and nothing is stored inside the loop (lane r keeps the result of
+// row r until one coalesced store at the end): only then does the compiler know how many requests
+// are outstanding at each wait and leaves the younger ones in flight.
 
 // Activation pieces (8 values) a thread stages: piece p = threadIdx.x + i*256 of MT*PIECES_PER_ROW.
 template <typename CT, int MT, int kPiecesPerRow>
@@ -319,7 +338,7 @@ __device__ __forceinline__ void x_request(const RowArgs &a, XPieces<CT, MT, kPie
     const int m = p / kPiecesPerRow;
     const int piece = p - m * kPiecesPerRow;
     const int msrc = m < a.M ? m : a.M - 1;
-    if (p < MT * kPiecesPerRow)
+    if (XPieces<CT, MT, kPiecesPerRow>::kTotal % 256 == 0 || p < MT * kPiecesPerRow)
       xp.v[i] = *reinterpret_cast<const vec_t *>(xg + static_cast<int64_t>(msrc) * a.K + piece * 8);
   }
 }
@@ -333,7 +352,7 @@ __device__ __forceinline__ void x_commit(const XPieces<CT, MT, kPiecesPerRow> &x
 #pragma unroll
   for (int i = 0; i < XPieces<CT, MT, kPiecesPerRow>::kPerThread; ++i) {
     const int p = threadIdx.x + i * 256;
-    if (p < MT * kPiecesPerRow) {
+    if (XPieces<CT, MT, kPiecesPerRow>::kTotal % 256 == 0 || p < MT * kPiecesPerRow) {
       const int m = p / kPiecesPerRow;
       const int piece = p - m * kPiecesPerRow;
       vec_t v = xp.v[i];
@@ -366,7 +385,7 @@ template <typename CT, int MT, int CPR>
 __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
 {
   typedef typename Mfma16<CT>::vec_t vec_t;
-  constexpr int D = (CPR >= 4) ? 1 : 4 / CPR;   // rows in flight (measured best: 4 loads per lane)
+  constexpr int D = (CPR >= 2) ? 2 : 4;   // rows in the ring (2 for K = 4096 measured best against 1, 3, 4 and 8)
   constexpr int kPieces = CPR * 256;         // 8-value pieces per activation row
   constexpr int kGroupsPad = CPR * 16;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -391,16 +410,24 @@ __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
   const f16_t *sp = static_cast<const f16_t *>(a.scales) + row0 * groups_per_row;
   u32x4_t w[D][CPR];
   f16_t sc[D][CPR];
+  // Every load below is issued unconditionally (a row index past the wave's range reads the start of
+  // the activation row instead, which is cache resident and large enough): with no branch around a
+  // load the compiler knows how many requests are in flight at every wait and lets the newer ones
+  // stay outstanding, which is what keeps the ring of rows in flight.
+  const uint8_t *wdummy = static_cast<const uint8_t *>(a.x) + pslot * 16;
+  const f16_t *sdummy = static_cast<const f16_t *>(a.x) + di;
   auto issue = [&](int d, int r) {
+    const bool ok = r < nrows;
+    const uint8_t *wsrc = ok ? wp + r * kRowBytes : wdummy;
+    const f16_t *ssrc = ok ? sp + r * groups_per_row + di : sdummy;
 #pragma unroll
     for (int c = 0; c < CPR; ++c) {
-      w[d][c] = *reinterpret_cast<const u32x4_t *>(wp + r * kRowBytes + c * 1024);
-      sc[d][c] = sp[r * groups_per_row + c * 16 + di];
+      w[d][c] = *reinterpret_cast<const u32x4_t *>(wsrc + c * 1024);
+      sc[d][c] = ssrc[c * 16];
     }
   };
 #pragma unroll
-  for (int d = 0; d < D; ++d)
-    if (d < nrows) issue(d, d);
+  for (int d = 0; d < D; ++d) issue(d, d);
 
   x_commit<CT, MT, kPieces, true>(xp, xs, xsum);
   __syncthreads();
@@ -411,20 +438,17 @@ __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
 #pragma unroll
     for (int c = 0; c < CPR; ++c) corr[m][c] = Mfma16<CT>::kOffset * xsum[m * kGroupsPad + c * 16 + di];
   const int tsel = di & 3;
+  // lane r keeps the result of the wave's row r: one coalesced store per wave after the loop, and no
+  // store (which would count against the same in-flight counter as the loads) inside it
+  float res[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) res[m] = 0.0f;
 
   for (int r0 = 0; r0 < nrows; r0 += D) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
       const int r = r0 + d;
       if (r < nrows) {
-        u32x4_t wr[CPR];
-        float sr[CPR];
-#pragma unroll
-        for (int c = 0; c < CPR; ++c) {
-          wr[c] = w[d][c];
-          sr[c] = to_f32(sc[d][c]);
-        }
-        if (r + D < nrows) issue(d, r + D);
         float tot[MT];
 #pragma unroll
         for (int m = 0; m < MT; ++m) tot[m] = 0.0f;
@@ -436,11 +460,14 @@ __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             u32x4_t c4;
-            const uint32_t p = wr[c][j];
-            c4[0] = (p & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
-            c4[1] = ((p >> 4) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
-            c4[2] = ((p >> 8) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
-            c4[3] = ((p >> 12) & 0x000F000Fu) ^ Mfma16<CT>::kMagic;
+            // one xor turns all eight two's-complement nibbles into code + 8; each pair of nibbles then
+            // needs a shift and one and-or to become two compute-dtype values 128 (or 1024) + code + 8
+            const uint32_t p = w[d][c][j] ^ 0x88888888u;
+            constexpr uint32_t kBase = Mfma16<CT>::kMagic & 0xFFF0FFF0u;
+            c4[0] = and_or(p, 0x000F000Fu, kBase);
+            c4[1] = and_or(p >> 4, 0x000F000Fu, kBase);
+            c4[2] = and_or(p >> 8, 0x000F000Fu, kBase);
+            c4[3] = and_or(p >> 12, 0x000F000Fu, kBase);
             const vec_t av = *reinterpret_cast<const vec_t *>(&c4);
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
@@ -454,16 +481,22 @@ __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
             dsel = (tsel == 1) ? part[m][1] : dsel;
             dsel = (tsel == 2) ? part[m][2] : dsel;
             dsel = (tsel == 3) ? part[m][3] : dsel;
-            tot[m] = __builtin_fmaf(sr[c], dsel - corr[m][c], tot[m]);
+            tot[m] = __builtin_fmaf(to_f32(sc[d][c]), dsel - corr[m][c], tot[m]);
           }
         }
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
           const float v = wave_sum_hi(is_diag ? tot[m] : 0.0f);
-          if (lane == 63 && (MT != 4 || m < a.M)) static_cast<float *>(a.y)[static_cast<int64_t>(m) * a.N + row0 + r] = v;
+          res[m] = lane_insert(res[m], v, r);
         }
       }
+      issue(d, r + D);      // into the registers just consumed: the other D-1 rows stay in flight meanwhile
     }
+  }
+  if (lane < nrows) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+      if (MT != 4 || m < a.M) static_cast<float *>(a.y)[static_cast<int64_t>(m) * a.N + row0 + lane] = res[m];
   }
 }
 
@@ -471,7 +504,7 @@ template <typename CT, int MT, bool kVec, int CPR>
 __global__ __launch_bounds__(256) void rowlin_int8_fast_kernel(RowArgs a)
 {
   typedef typename Mfma16<CT>::vec_t vec_t;
-  constexpr int D = (CPR >= 4) ? 1 : 4 / CPR;   // rows in flight
+  constexpr int D = (CPR >= 4) ? 2 : 4;   // rows in the ring
   constexpr int kPieces = CPR * 128;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   CT *xs = reinterpret_cast<CT *>(smem);     // [MT][CPR*1024]
@@ -495,24 +528,13 @@ __global__ __launch_bounds__(256) void rowlin_int8_fast_kernel(RowArgs a)
   XPieces<CT, MT, kPieces> xp;
   x_request<CT, MT, kPieces>(a, xp);
 
-  const uint8_t *wp = a.wq + (cls + V * i0) * kRowBytes + lane * 16;
-  const int64_t rstep = V * kRowBytes;
-  u32x4_t w[D][CPR];
-  auto issue = [&](int d, int r) {
-#pragma unroll
-    for (int c = 0; c < CPR; ++c) w[d][c] = *reinterpret_cast<const u32x4_t *>(wp + r * rstep + c * 1024);
-  };
-#pragma unroll
-  for (int d = 0; d < D; ++d)
-    if (d < nrows) issue(d, d);
-
   floatx4_t sc[CPR][4];
   float s_scalar = 1.0f;
   if constexpr (kVec) {
     const float *sp = static_cast<const float *>(a.scales);
 #pragma unroll
     for (int c = 0; c < CPR; ++c) {
-      const int idx = static_cast<int>((static_cast<int64_t>(cls) * (CPR * 1024) + (c * 64 + lane) * 16) % a.period);
+      const int idx = static_cast<int>((static_cast<uint32_t>(cls) * (CPR * 1024) + (c * 64 + lane) * 16) % static_cast<uint32_t>(a.period));
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         int i = idx + 4 * q;
@@ -524,18 +546,31 @@ __global__ __launch_bounds__(256) void rowlin_int8_fast_kernel(RowArgs a)
     if (a.scales) s_scalar = static_cast<const float *>(a.scales)[0];
   }
 
+  // unconditional loads (a row past the wave's range reads the start of the activation row): see the
+  // int4 kernel above
+  const uint8_t *wp = a.wq + (cls + V * i0) * kRowBytes + lane * 16;
+  const uint8_t *wdummy = static_cast<const uint8_t *>(a.x) + lane * 16;
+  const int64_t rstep = V * kRowBytes;
+  u32x4_t w[D][CPR];
+  auto issue = [&](int d, int r) {
+    const uint8_t *wsrc = r < nrows ? wp + r * rstep : wdummy;
+#pragma unroll
+    for (int c = 0; c < CPR; ++c) w[d][c] = *reinterpret_cast<const u32x4_t *>(wsrc + c * 1024);
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d) issue(d, d);
+
   x_commit<CT, MT, kPieces, false>(xp, xs, nullptr);
   __syncthreads();
 
+  float res[MT];             // lane r: results of the wave's row r
+#pragma unroll
+  for (int m = 0; m < MT; ++m) res[m] = 0.0f;
   for (int r0 = 0; r0 < nrows; r0 += D) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
       const int r = r0 + d;
       if (r < nrows) {
-        u32x4_t wr[CPR];
-#pragma unroll
-        for (int c = 0; c < CPR; ++c) wr[c] = w[d][c];
-        if (r + D < nrows) issue(d, r + D);
         floatx4_t acc[MT];
 #pragma unroll
         for (int m = 0; m < MT; ++m) acc[m] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
@@ -544,8 +579,8 @@ __global__ __launch_bounds__(256) void rowlin_int8_fast_kernel(RowArgs a)
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
             float lo[4], hi[4];
-            int8x4_to_f32(wr[c][2 * j], lo);
-            int8x4_to_f32(wr[c][2 * j + 1], hi);
+            int8x4_to_f32(w[d][c][2 * j], lo);
+            int8x4_to_f32(w[d][c][2 * j + 1], hi);
             vec_t av;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -561,14 +596,19 @@ __global__ __launch_bounds__(256) void rowlin_int8_fast_kernel(RowArgs a)
             }
           }
         }
-        const int64_t nrow = cls + V * (i0 + r);
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
           const float v = wave_sum_hi(diag_of(acc[m], lane));
-          if (lane == 63 && (MT != 4 || m < a.M)) static_cast<float *>(a.y)[static_cast<int64_t>(m) * a.N + nrow] = v;
+          res[m] = lane_insert(res[m], v, r);
         }
       }
+      issue(d, r + D);
     }
+  }
+  if (lane < nrows) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+      if (MT != 4 || m < a.M) static_cast<float *>(a.y)[static_cast<int64_t>(m) * a.N + cls + V * (i0 + lane)] = res[m];
   }
 }
 
@@ -589,7 +629,7 @@ typedef int i32x4_t __attribute__((ext_vector_type(4)));
 template <typename XT, bool kVec, int CPR>
 __global__ __launch_bounds__(256) void rowlin_int8_digits_kernel(RowArgs a)
 {
-  constexpr int D = (CPR >= 4) ? 1 : 4 / CPR;   // rows in flight (4 loads per lane measured best)
+  constexpr int D = (CPR >= 4) ? 2 : 4;   // rows in the ring (2 for K = 4096 measured best against 1 and 4)
   __shared__ float mx[4][16];                                  // per chunk: max |x'| of every diagonal element
   __shared__ __attribute__((aligned(16))) i32x4_t dig[4][3][64];   // [chunk][digit][lane]
 
@@ -609,39 +649,53 @@ __global__ __launch_bounds__(256) void rowlin_int8_digits_kernel(RowArgs a)
   }
   constexpr int64_t kRowBytes = static_cast<int64_t>(CPR) * 1024;
 
-  // this lane's activations of chunk `wave` (chunks beyond CPR do not exist; their waves only join the barriers)
+  // this lane's activations of chunk `wave` (chunks beyond CPR do not exist; their waves only join the
+  // barriers) and their scales are requested BEFORE the first weight rows: loads return in order, so
+  // everything the prologue needs must be ahead of the long HBM latency of the weights in the queue
   float xv[16];
+  floatx4_t scv[4];
   const bool has_chunk = wave < CPR;
   if (has_chunk) {
     const XT *xg = static_cast<const XT *>(a.x) + (wave * 64 + lane) * 16;
 #pragma unroll
     for (int t = 0; t < 16; ++t) xv[t] = to_f32<XT>(xg[t]);
+    if constexpr (kVec) {
+      const float *sp = static_cast<const float *>(a.scales);
+      // 32-bit arithmetic: cls < N / 256 and K <= 4096, so cls * K + k stays far below 2^31
+      const int idx = static_cast<int>((static_cast<uint32_t>(cls) * (CPR * 1024) + (wave * 64 + lane) * 16) % static_cast<uint32_t>(a.period));
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        int i = idx + 4 * q;
+        if (i >= a.period) i -= a.period;
+        scv[q] = *reinterpret_cast<const floatx4_t *>(sp + i);
+      }
+    }
+  }
+  float s_scalar = 1.0f;
+  if constexpr (!kVec) {
+    if (a.scales) s_scalar = static_cast<const float *>(a.scales)[0];
   }
 
   const uint8_t *wp = a.wq + (cls + V * i0) * kRowBytes + lane * 16;
   const int64_t rstep = V * kRowBytes;
   i32x4_t w[D][CPR];
+  // unconditional loads (a row past the wave's range reads the start of the activation row): see the
+  // int4 kernel above
+  const uint8_t *wdummy = static_cast<const uint8_t *>(a.x) + lane * 16;
   auto issue = [&](int d, int r) {
+    const uint8_t *wsrc = r < nrows ? wp + r * rstep : wdummy;
 #pragma unroll
-    for (int c = 0; c < CPR; ++c) w[d][c] = *reinterpret_cast<const i32x4_t *>(wp + r * rstep + c * 1024);
+    for (int c = 0; c < CPR; ++c) w[d][c] = *reinterpret_cast<const i32x4_t *>(wsrc + c * 1024);
   };
 #pragma unroll
-  for (int d = 0; d < D; ++d)
-    if (d < nrows) issue(d, d);
+  for (int d = 0; d < D; ++d) issue(d, d);
 
-  float s_scalar = 1.0f;
   if (has_chunk) {
     if constexpr (kVec) {
-      const float *sp = static_cast<const float *>(a.scales);
-      const int idx = static_cast<int>((static_cast<int64_t>(cls) * (CPR * 1024) + (wave * 64 + lane) * 16) % a.period);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        int i = idx + 4 * q;
-        if (i >= a.period) i -= a.period;
-        const floatx4_t sc = *reinterpret_cast<const floatx4_t *>(sp + i);
+      for (int q = 0; q < 4; ++q)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) xv[4 * q + t] *= sc[t];
-      }
+        for (int t = 0; t < 4; ++t) xv[4 * q + t] *= scv[q][t];
     }
     float m = 0.0f;
 #pragma unroll
@@ -649,9 +703,6 @@ __global__ __launch_bounds__(256) void rowlin_int8_digits_kernel(RowArgs a)
     m = fmaxf(m, __shfl_xor(m, 16));
     m = fmaxf(m, __shfl_xor(m, 32));
     if (lane < 16) mx[wave][lane] = m;
-  }
-  if constexpr (!kVec) {
-    if (a.scales) s_scalar = static_cast<const float *>(a.scales)[0];
   }
   __syncthreads();
 
@@ -700,21 +751,18 @@ __global__ __launch_bounds__(256) void rowlin_int8_digits_kernel(RowArgs a)
   const int tsel = lane & 3;
   const bool is_diag = (lane >> 4) == ((lane & 15) >> 2);
 
+  float res = 0.0f;          // lane r: result of the wave's row r
   for (int r0 = 0; r0 < nrows; r0 += D) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
       const int r = r0 + d;
       if (r < nrows) {
-        i32x4_t wr[CPR];
-#pragma unroll
-        for (int c = 0; c < CPR; ++c) wr[c] = w[d][c];
-        if (r + D < nrows) issue(d, r + D);
         i32x4_t s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0}, s2 = {0, 0, 0, 0};
 #pragma unroll
         for (int c = 0; c < CPR; ++c) {
-          s0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[c], xb[c][0], s0, 0, 0, 0);
-          s1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[c], xb[c][1], s1, 0, 0, 0);
-          s2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[c], xb[c][2], s2, 0, 0, 0);
+          s0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[d][c], xb[c][0], s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[d][c], xb[c][1], s1, 0, 0, 0);
+          s2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[d][c], xb[c][2], s2, 0, 0, 0);
         }
         // D[i][i] sits in element i%4 of lane i + 16*(i/4)
         int p0 = s0[0], p1 = s1[0], p2 = s2[0];
@@ -725,10 +773,12 @@ __global__ __launch_bounds__(256) void rowlin_int8_digits_kernel(RowArgs a)
         v = __builtin_fmaf(static_cast<float>(p1), u1, v);
         v = __builtin_fmaf(static_cast<float>(p2), u2, v);
         v = wave_sum_hi(is_diag ? v : 0.0f);
-        if (lane == 63) static_cast<float *>(a.y)[cls + V * (i0 + r)] = v;
+        res = lane_insert(res, v, r);
       }
+      issue(d, r + D);
     }
   }
+  if (lane < nrows) static_cast<float *>(a.y)[cls + V * (i0 + lane)] = res;
 }
 
 
