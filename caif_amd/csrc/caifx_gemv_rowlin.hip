@@ -28,6 +28,8 @@
 //     the codes go into the integer matrix core as loaded (rowlin_int8_digits_kernel below).
 #include "caifx_internal.hpp"
 
+#include <atomic>
+
 namespace caifx {
 namespace {
 
@@ -126,6 +128,14 @@ __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t b
   uint32_t r;
   asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(base));
   return r;
+}
+
+// the low bytes of four words as one word (a in byte 0)
+__device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d)
+{
+  const uint32_t ab = __builtin_amdgcn_perm(static_cast<uint32_t>(b), static_cast<uint32_t>(a), 0x0c0c0400u);
+  const uint32_t cd = __builtin_amdgcn_perm(static_cast<uint32_t>(d), static_cast<uint32_t>(c), 0x0c0c0400u);
+  return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
 }
 
 // `acc` with lane `dst_lane` (wave uniform) replaced by the wave sum that wave_sum_hi left in lane 63
@@ -319,40 +329,40 @@ __global__ __launch_bounds__(256) void rowlin_int4_kernel(RowArgs a)
 // row r until one coalesced store at the end): only then does the compiler know how many requests
 // are outstanding at each wait and leaves the younger ones in flight.
 
-// Activation pieces (8 values) a thread stages: piece p = threadIdx.x + i*256 of MT*PIECES_PER_ROW.
-template <typename CT, int MT, int kPiecesPerRow>
+// Activation pieces (8 values) a thread stages: piece p = threadIdx.x + i*kThreads of MT*PIECES_PER_ROW.
+template <typename CT, int MT, int kPiecesPerRow, int kThreads = 256>
 struct XPieces {
   static constexpr int kTotal = MT * kPiecesPerRow;
-  static constexpr int kPerThread = (kTotal + 255) / 256;
+  static constexpr int kPerThread = (kTotal + kThreads - 1) / kThreads;
   typename Mfma16<CT>::vec_t v[kPerThread];
 };
 
-template <typename CT, int MT, int kPiecesPerRow>
-__device__ __forceinline__ void x_request(const RowArgs &a, XPieces<CT, MT, kPiecesPerRow> &xp)
+template <typename CT, int MT, int kPiecesPerRow, int kThreads = 256>
+__device__ __forceinline__ void x_request(const RowArgs &a, XPieces<CT, MT, kPiecesPerRow, kThreads> &xp)
 {
   typedef typename Mfma16<CT>::vec_t vec_t;
   const CT *xg = static_cast<const CT *>(a.x);
 #pragma unroll
-  for (int i = 0; i < XPieces<CT, MT, kPiecesPerRow>::kPerThread; ++i) {
-    const int p = threadIdx.x + i * 256;
+  for (int i = 0; i < XPieces<CT, MT, kPiecesPerRow, kThreads>::kPerThread; ++i) {
+    const int p = threadIdx.x + i * kThreads;
     const int m = p / kPiecesPerRow;
     const int piece = p - m * kPiecesPerRow;
     const int msrc = m < a.M ? m : a.M - 1;
-    if (XPieces<CT, MT, kPiecesPerRow>::kTotal % 256 == 0 || p < MT * kPiecesPerRow)
+    if (XPieces<CT, MT, kPiecesPerRow, kThreads>::kTotal % kThreads == 0 || p < MT * kPiecesPerRow)
       xp.v[i] = *reinterpret_cast<const vec_t *>(xg + static_cast<int64_t>(msrc) * a.K + piece * 8);
   }
 }
 
-template <typename CT, int MT, int kPiecesPerRow, bool kInt4>
-__device__ __forceinline__ void x_commit(const XPieces<CT, MT, kPiecesPerRow> &xp, CT *xs, float *xsum)
+template <typename CT, int MT, int kPiecesPerRow, bool kInt4, int kThreads = 256>
+__device__ __forceinline__ void x_commit(const XPieces<CT, MT, kPiecesPerRow, kThreads> &xp, CT *xs, float *xsum)
 {
   typedef typename Mfma16<CT>::vec_t vec_t;
   constexpr int kSteps = kInt4 ? 4 : 2;
   const int lane = threadIdx.x & 63;
 #pragma unroll
-  for (int i = 0; i < XPieces<CT, MT, kPiecesPerRow>::kPerThread; ++i) {
-    const int p = threadIdx.x + i * 256;
-    if (XPieces<CT, MT, kPiecesPerRow>::kTotal % 256 == 0 || p < MT * kPiecesPerRow) {
+  for (int i = 0; i < XPieces<CT, MT, kPiecesPerRow, kThreads>::kPerThread; ++i) {
+    const int p = threadIdx.x + i * kThreads;
+    if (XPieces<CT, MT, kPiecesPerRow, kThreads>::kTotal % kThreads == 0 || p < MT * kPiecesPerRow) {
       const int m = p / kPiecesPerRow;
       const int piece = p - m * kPiecesPerRow;
       vec_t v = xp.v[i];
@@ -381,9 +391,12 @@ __device__ __forceinline__ void x_commit(const XPieces<CT, MT, kPiecesPerRow> &x
   }
 }
 
+constexpr int kInt4FastWaves = 4;   // waves per workgroup of the kernel below (8 and 16 measured no better)
+
 template <typename CT, int MT, int CPR>
-__global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
+__global__ __launch_bounds__(kInt4FastWaves * 64) void rowlin_int4_fast_kernel(RowArgs a)
 {
+  constexpr int kThreads = kInt4FastWaves * 64;
   typedef typename Mfma16<CT>::vec_t vec_t;
   constexpr int D = (CPR >= 2) ? 2 : 4;   // rows in the ring (2 for K = 4096 measured best against 1, 3, 4 and 8)
   constexpr int kPieces = CPR * 256;         // 8-value pieces per activation row
@@ -394,7 +407,7 @@ __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * a.rows_per_wave;
+  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * kInt4FastWaves + wave) * a.rows_per_wave;
   int nrows = 0;
   if (row0 < a.N) nrows = static_cast<int>(a.N - row0 < a.rows_per_wave ? a.N - row0 : a.rows_per_wave);
   const bool is_diag = (lane >> 4) == ((lane & 15) >> 2);
@@ -403,8 +416,8 @@ __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
   constexpr int64_t kRowBytes = static_cast<int64_t>(CPR) * 1024;
   constexpr int groups_per_row = CPR * 16;       // group size 128
 
-  XPieces<CT, MT, kPieces> xp;
-  x_request<CT, MT, kPieces>(a, xp);
+  XPieces<CT, MT, kPieces, kThreads> xp;
+  x_request<CT, MT, kPieces, kThreads>(a, xp);
 
   const uint8_t *wp = a.wq + row0 * kRowBytes + pslot * 16;
   const f16_t *sp = static_cast<const f16_t *>(a.scales) + row0 * groups_per_row;
@@ -429,7 +442,7 @@ __global__ __launch_bounds__(256) void rowlin_int4_fast_kernel(RowArgs a)
 #pragma unroll
   for (int d = 0; d < D; ++d) issue(d, d);
 
-  x_commit<CT, MT, kPieces, true>(xp, xs, xsum);
+  x_commit<CT, MT, kPieces, true, kThreads>(xp, xs, xsum);
   __syncthreads();
 
   float corr[MT][CPR];
@@ -626,8 +639,13 @@ __global__ __launch_bounds__(256) void rowlin_int8_fast_kernel(RowArgs a)
 // of q*scale to the compute dtype that the reference applies and this kernel does not.
 typedef int i32x4_t __attribute__((ext_vector_type(4)));
 
+// Waves per workgroup of the kernel below.  The prologue (activations times scales, digit planes) is
+// paid once per workgroup and reads 24 KB for K = 4096, so a workgroup should own many rows: 16 waves
+// measured 12.2 us against 12.9 (8) and 13.1 (4) on the K=4096, N=14336 case.
+constexpr int kDigitWaves = 16;
+
 template <typename XT, bool kVec, int CPR>
-__global__ __launch_bounds__(256) void rowlin_int8_digits_kernel(RowArgs a)
+__global__ __launch_bounds__(kDigitWaves * 64) void rowlin_int8_digits_kernel(RowArgs a)
 {
   constexpr int D = (CPR >= 4) ? 2 : 4;   // rows in the ring (2 for K = 4096 measured best against 1 and 4)
   __shared__ float mx[4][16];                                  // per chunk: max |x'| of every diagonal element
@@ -635,8 +653,8 @@ __global__ __launch_bounds__(256) void rowlin_int8_digits_kernel(RowArgs a)
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int gw = blockIdx.x * 4 + wave;
-  const int cls = (blockIdx.x * 4) / a.waves_per_class;        // waves_per_class is a multiple of 4: one class per workgroup
+  const int gw = blockIdx.x * kDigitWaves + wave;
+  const int cls = (blockIdx.x * kDigitWaves) / a.waves_per_class;        // waves_per_class is a multiple of kDigitWaves: one class per workgroup
   const int64_t i0 = static_cast<int64_t>(gw - cls * a.waves_per_class) * a.rows_per_wave;
   const int64_t V = a.row_stride;
   int nrows = 0;
@@ -717,25 +735,24 @@ __global__ __launch_bounds__(256) void rowlin_int8_digits_kernel(RowArgs a)
     unit = m > 0.0f ? ldexpf(1.0f, e - 6) : 1.0f;
   }
   if (has_chunk) {
-    const float inv = 1.0f / unit;            // exact: a power of two
+    // n = round(x' / unit * 2^14) as the low mantissa bits of x' * (2^14 / unit) + 1.5 * 2^23 (|n| <= 2^20);
+    // n = 2^14 d0 + 2^7 d1 + d2 with d1, d2 in [-64, 63]: three signed bit-field extracts, the carries
+    // supplied by adding half a digit below each field
+    const float inv14 = 16384.0f / unit;      // exact: a power of two
     i32x4_t d0, d1, d2;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      uint32_t b0 = 0, b1 = 0, b2 = 0;
+      int e0[4], e1[4], e2[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const float v = xv[4 * q + t] * inv;           // |v| <= 64
-        const float r0 = rintf(v);
-        const float v1 = (v - r0) * 128.0f;            // exact, |v1| <= 64
-        const float r1 = rintf(v1);
-        const float r2 = rintf((v1 - r1) * 128.0f);
-        b0 |= (static_cast<uint32_t>(static_cast<int>(r0)) & 0xFFu) << (8 * t);
-        b1 |= (static_cast<uint32_t>(static_cast<int>(r1)) & 0xFFu) << (8 * t);
-        b2 |= (static_cast<uint32_t>(static_cast<int>(r2)) & 0xFFu) << (8 * t);
+        const int b = __builtin_bit_cast(int, __builtin_fmaf(xv[4 * q + t], inv14, 12582912.0f));
+        e2[t] = __builtin_amdgcn_sbfe(b, 0, 7);
+        e1[t] = __builtin_amdgcn_sbfe(b + 64, 7, 7);
+        e0[t] = __builtin_amdgcn_sbfe(b + 64 + 8192, 14, 8);
       }
-      d0[q] = static_cast<int>(b0);
-      d1[q] = static_cast<int>(b1);
-      d2[q] = static_cast<int>(b2);
+      d0[q] = static_cast<int>(pack_low_bytes(e0[0], e0[1], e0[2], e0[3]));
+      d1[q] = static_cast<int>(pack_low_bytes(e1[0], e1[1], e1[2], e1[3]));
+      d2[q] = static_cast<int>(pack_low_bytes(e2[0], e2[1], e2[2], e2[3]));
     }
     dig[wave][0][lane] = d0;
     dig[wave][1][lane] = d1;
@@ -898,8 +915,9 @@ template <typename CT, int MT, int CPR>
 int launch_int4_fast(const RowArgs &ra, hipStream_t s)
 {
   const size_t lds = static_cast<size_t>((MT * CPR * 16 + 3) & ~3) * 4 + static_cast<size_t>(MT) * CPR * 2048 * 2;
-  hipLaunchKernelGGL((rowlin_int4_fast_kernel<CT, MT, CPR>), dim3(static_cast<unsigned>((ra.total_waves + 3) / 4)),
-                     dim3(256), lds, s, ra);
+  hipLaunchKernelGGL((rowlin_int4_fast_kernel<CT, MT, CPR>),
+                     dim3(static_cast<unsigned>((ra.total_waves + kInt4FastWaves - 1) / kInt4FastWaves)), dim3(kInt4FastWaves * 64),
+                     lds, s, ra);
   return launch_status();
 }
 
@@ -930,7 +948,7 @@ int launch_int4(const RowArgs &ra, hipStream_t s)
 template <typename XT, bool kVec, int CPR>
 int launch_int8_digits(const RowArgs &ra, hipStream_t s)
 {
-  hipLaunchKernelGGL((rowlin_int8_digits_kernel<XT, kVec, CPR>), dim3(static_cast<unsigned>(ra.total_waves / 4)), dim3(256), 0, s, ra);
+  hipLaunchKernelGGL((rowlin_int8_digits_kernel<XT, kVec, CPR>), dim3(static_cast<unsigned>(ra.total_waves / kDigitWaves)), dim3(kDigitWaves * 64), 0, s, ra);
   return launch_status();
 }
 
@@ -998,6 +1016,18 @@ int64_t gcd64(int64_t a, int64_t b)
   return a;
 }
 
+int64_t compute_unit_count()
+{
+  static std::atomic<int> cached{0};
+  int n = cached.load(std::memory_order_relaxed);
+  if (n == 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached.store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
 int pick_rows_per_wave(int64_t rows, int min_rows, int64_t target = 2048)
 {
   // aim for two waves per SIMD (2048 waves): each walks its rows through a ring of loads, so
@@ -1060,10 +1090,17 @@ int rowlin_forward(const GemmArgs &g, hipStream_t s)
     const bool digits = g.M == 1 && g.K % 1024 == 0 && (ra.cpr == 1 || ra.cpr == 2 || ra.cpr == 4) && g.y_dtype == CAIFX_F32;
     // the integer-matrix-core kernel is light on registers and arithmetic: four waves per SIMD measured best
     ra.rows_per_wave = digits ? pick_rows_per_wave(g.N, 1, 4096) : pick_rows_per_wave(g.N, kind == 2 ? 2 * rb : rb);
+    if (digits) {
+      // one workgroup per compute unit at a time (16 waves): keep the grid within one round when the rows allow
+      const int64_t cus = compute_unit_count();
+      while (ra.rows_per_wave < 64 &&
+             ra.row_stride * (((rows_class + ra.rows_per_wave - 1) / ra.rows_per_wave + kDigitWaves - 1) / kDigitWaves) > cus)
+        ++ra.rows_per_wave;
+    }
     ra.waves_per_class = static_cast<int>((rows_class + ra.rows_per_wave - 1) / ra.rows_per_wave);
     if (digits) {
       ra.digits = 1;
-      ra.waves_per_class = (ra.waves_per_class + 3) / 4 * 4;      // a workgroup of 4 waves stays inside one class
+      ra.waves_per_class = (ra.waves_per_class + kDigitWaves - 1) / kDigitWaves * kDigitWaves;      // a workgroup stays inside one class
     }
     ra.total_waves = ra.waves_per_class * ra.row_stride;
     if (static_cast<size_t>(mt) * ra.xpitch * 2 > 64 * 1024) return CAIFX_ERR_UNSUPPORTED;
