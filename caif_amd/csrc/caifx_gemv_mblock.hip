@@ -13,11 +13,16 @@
 //         OFFSET' * sum(x) and multiplied by the group's scale ("post-scaling": the weight is never
 //         rounded to the compute dtype, so results differ from the dequantise-then-cast reference
 //         by that rounding, a few 1e-3 of the largest output);
-//   int8: 16 codes at k = group*128 + half*64 + q*16, each multiplied by its scale in fp32 and
-//         rounded once to the compute dtype, exactly as the reference forms its weight.  A scale
+//   int8: 16 codes at k = group*128 + half*64 + q*16, fed to v_mfma_i32_16x16x64_i8 exactly as loaded
+//         (no unpacking arithmetic).  The scales are folded into the activations instead: a scale
 //         vector of period P is addressed by the flat index n*K + k modulo P; rows n with equal
-//         n mod V, V = P / gcd(K mod P, P), see the same scales along k, so a workgroup only visits rows
-//         of one residue class and keeps that class's K scales in LDS.
+//         n mod V, V = P / gcd(K mod P, P), see the same scales along k, so a workgroup only visits
+//         rows of one residue class, stages that class's K scales in LDS once and forms
+//         x'[m][k] = x[m][k] * scale[k] in fp32.  x' is split into three signed 7-bit digit planes
+//         relative to a power-of-two unit per activation row and wave (x' ~ unit * (d0 + d1/128 +
+//         d2/16384), error <= unit * 2^-15); the three exact int32 sums are combined in fp32 per block.
+//         The weight is therefore never rounded to the compute dtype: results differ from the
+//         dequantise-then-cast reference by that rounding (a few 1e-3 of the largest output), like int4.
 // After the last group every wave holds a partial 16x16 tile; the 16 partials are added through LDS
 // in a fixed order (results do not depend on scheduling) and written as Y[token][row].
 #include "caifx_internal.hpp"
@@ -107,6 +112,16 @@ __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t b
   return r;
 }
 
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+
+// the low bytes of four words as one word (a in byte 0)
+__device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d)
+{
+  const uint32_t ab = __builtin_amdgcn_perm(static_cast<uint32_t>(b), static_cast<uint32_t>(a), 0x0c0c0400u);
+  const uint32_t cd = __builtin_amdgcn_perm(static_cast<uint32_t>(d), static_cast<uint32_t>(c), 0x0c0c0400u);
+  return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
+}
+
 constexpr int kSegBlocks = 16;                         // row blocks between two flushes of the output staging buffer
 constexpr int kSegRows = kSegBlocks * 16;
 
@@ -185,7 +200,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
   }
   // int8 scale vector of this residue class: svec[k] = scales[(cls*K + k) mod period], K <= 4096
   float s_one = 1.0f;
-  float sv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  float sv[4] = {1.0f, 1.0f, 1.0f, 1.0f};     // without a scale vector the staged scales are 1
   if constexpr (!kInt4) {
     if (a.period > 0) {
       int idx = static_cast<int>((static_cast<int64_t>(cls) * a.K + threadIdx.x) % a.period);
@@ -214,12 +229,10 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
     }
   }
   if constexpr (!kInt4) {
-    if (a.period > 0) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const int k = threadIdx.x + t * kMbThreads;
-        if (k < a.K) svec[k] = sv[t];
-      }
+    for (int t = 0; t < 4; ++t) {
+      const int k = threadIdx.x + t * kMbThreads;
+      if (k < a.K) svec[k] = sv[t];
     }
   }
 
@@ -250,7 +263,71 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
       for (int r = 0; r < 4; ++r) cor[g][r] = Mfma16<CT>::kOffset * xsum[r];
     }
   }
-  if constexpr (!kInt4) __syncthreads();       // svec is complete
+  // int8: digit planes of x' = x * scale as A operands of the integer matrix core, dg[step][plane];
+  // step t covers k = (g0 + t/2)*128 + (t%2)*64 + q*16 .. +16 of activation row j
+  constexpr int kSteps = 2 * GPW;
+  constexpr int kPlanes = 3;              // 2 would give 14-bit activations; the third plane costs 4 of 12 MFMAs per block
+  i32x4_t dg[kInt4 ? 1 : kSteps][kPlanes];
+  float ur[4] = {1.0f, 1.0f, 1.0f, 1.0f};     // unit of the activation rows 4q..4q+3 this lane holds results of
+  if constexpr (!kInt4) {
+    __syncthreads();       // svec is complete
+    // four consecutive x' values: quad c (0..3) of step t
+    auto xprime4 = [&](int t, int c, float (&v)[4]) {
+      const int g = t >> 1;
+      const int gg = g0 + g < a.groups ? g0 + g : a.groups - 1;
+      const vec_t xv = xa[g][2 * (t & 1) + (c >> 1)];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = to_f32<CT>(xv[4 * (c & 1) + i]);
+      const floatx4_t sc4 = *reinterpret_cast<const floatx4_t *>(svec + gg * 128 + (t & 1) * 64 + q * 16 + 4 * c);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] *= sc4[i];
+    };
+    float mx = 0.0f;
+#pragma unroll
+    for (int t = 0; t < kSteps; ++t)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        float v[4];
+        xprime4(t, c, v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fabsf(v[i]));
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));      // over the four k quarters: row j's largest |x'| in this wave's k range
+    int e = 0;
+    (void)frexpf(mx, &e);                     // mx = f * 2^e, f in [0.5, 1)
+    const float unit = mx > 0.0f ? ldexpf(1.0f, e - 6) : 1.0f;    // |x'| / unit <= 64
+    const float inv14 = 16384.0f / unit;      // exact: a power of two
+#pragma unroll
+    for (int t = 0; t < kSteps; ++t) {
+      // n = round(x' / unit * 2^14) as the low mantissa bits of x' * inv14 + 1.5 * 2^23 (|n| <= 2^20);
+      // n = 2^14 d0 + 2^7 d1 + d2 with d1, d2 in [-64, 63]
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        float v[4];
+        xprime4(t, c, v);
+        int e0[4], e1[4], e2[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int b = __builtin_bit_cast(int, __builtin_fmaf(v[i], kPlanes == 3 ? inv14 : inv14 * (1.0f / 128.0f), 12582912.0f));
+          if constexpr (kPlanes == 3) {
+            e2[i] = __builtin_amdgcn_sbfe(b, 0, 7);
+            e1[i] = __builtin_amdgcn_sbfe(b + 64, 7, 7);
+            e0[i] = __builtin_amdgcn_sbfe(b + 64 + 8192, 14, 8);
+          } else {
+            e2[i] = 0;
+            e1[i] = __builtin_amdgcn_sbfe(b, 0, 7);
+            e0[i] = __builtin_amdgcn_sbfe(b + 64, 7, 8);
+          }
+        }
+        dg[t][0][c] = static_cast<int>(pack_low_bytes(e0[0], e0[1], e0[2], e0[3]));
+        dg[t][1][c] = static_cast<int>(pack_low_bytes(e1[0], e1[1], e1[2], e1[3]));
+        if constexpr (kPlanes == 3) dg[t][2][c] = static_cast<int>(pack_low_bytes(e2[0], e2[1], e2[2], e2[3]));
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) ur[r] = __shfl(unit, 4 * q + r) * s_one;
+  }
 
   // The waves run freely through RBB blocks of 16 rows (no barrier in between, so one wave's
   // arithmetic overlaps another's wait for HBM), then the 16 partial tiles of each block are added
@@ -285,28 +362,23 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
               const float sr = to_f32(sc[d][g]);
 #pragma unroll
               for (int r = 0; r < 4; ++r) tot[u][r] = __builtin_fmaf(sr, acc[r] - cor[g][r], tot[u][r]);
-            } else {
-              const int gg = g0 + g < a.groups ? g0 + g : a.groups - 1;
+            }
+          }
+          if constexpr (!kInt4) {
+            i32x4_t s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0}, s2 = {0, 0, 0, 0};
 #pragma unroll
-              for (int t = 0; t < 4; ++t) {
-                float lo[4], hi[4];
-                int8x4_to_f32(w[d][2 * g + (t >> 1)][2 * (t & 1)], lo);
-                int8x4_to_f32(w[d][2 * g + (t >> 1)][2 * (t & 1) + 1], hi);
-                floatx4_t s0 = {s_one, s_one, s_one, s_one};
-                floatx4_t s1 = s0;
-                if (a.period > 0) {
-                  const float *sp = svec + gg * 128 + (t >> 1) * 64 + q * 16 + 8 * (t & 1);
-                  s0 = *reinterpret_cast<const floatx4_t *>(sp);
-                  s1 = *reinterpret_cast<const floatx4_t *>(sp + 4);
-                }
-                vec_t bv;
+            for (int t = 0; t < kSteps; ++t) {
+              const i32x4_t bw = __builtin_bit_cast(i32x4_t, w[d][t]);
+              s0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[t][0], bw, s0, 0, 0, 0);
+              s1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[t][1], bw, s1, 0, 0, 0);
+              if constexpr (kPlanes == 3) s2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[t][2], bw, s2, 0, 0, 0);
+            }
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                  bv[i] = from_f32<CT>(lo[i] * s0[i]);
-                  bv[4 + i] = from_f32<CT>(hi[i] * s1[i]);
-                }
-                tot[u] = Mfma16<CT>::run(xa[g][t], bv, tot[u]);
-              }
+            for (int r = 0; r < 4; ++r) {
+              float v = static_cast<float>(s0[r]);
+              v = __builtin_fmaf(static_cast<float>(s1[r]), 1.0f / 128.0f, v);
+              if constexpr (kPlanes == 3) v = __builtin_fmaf(static_cast<float>(s2[r]), 1.0f / 16384.0f, v);
+              tot[u][r] = v * ur[r];
             }
           }
         }
@@ -417,8 +489,8 @@ int mblock_forward(const GemmArgs &g, hipStream_t s)
     m.period = static_cast<int>(P);
     m.scale_step = static_cast<int>(kMbThreads % P);
     m.V = static_cast<int>(V);
-    lds += static_cast<size_t>(g.K) * sizeof(float);
   }
+  if (!int4) lds += static_cast<size_t>(g.K) * sizeof(float);      // staged scales (ones without a scale vector)
   int target = compute_units();
   const int64_t nrb_class = ((g.N + m.V - 1) / m.V + 15) / 16;
   int64_t bpc = target / m.V;
