@@ -27,7 +27,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 K_DEC, N_DEC = 4096, 14336
-MEASURED_TRAFFIC_INT8_M1 = 59394850     # bytes per launch, rocprofv3 counters (see the roofline object)
+MEASURED_TRAFFIC_INT8_M1 = 59406822     # bytes per launch, rocprofv3 counters (see the roofline object)
 
 
 def algorithmic_bytes(kind, M, N=N_DEC, K=K_DEC, group=128):
@@ -167,7 +167,7 @@ def main():
         "avg_launch_us": round(per[dom]["us"], 3),
         "algorithmic_bytes_per_launch": algorithmic_bytes("int8", 1),
         # HBM bytes per launch of this kernel from two rocprofv3 --pmc runs (FETCH_SIZE x 1.9997 and
-        # WRITE_SIZE x 1.0000, factors from a plain 256 MiB copy in the same runs): 59.34 MB read +
+        # WRITE_SIZE x 1.0000, factors from a plain 256 MiB copy in the same runs): 59.35 MB read +
         # 0.06 MB written; the summary is profiles/decode_gemv_hbm_traffic.md
         "traffic": MEASURED_TRAFFIC_INT8_M1,
     }
