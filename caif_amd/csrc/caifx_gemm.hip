@@ -127,10 +127,30 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
   const uint8_t *wq = static_cast<const uint8_t *>(g.wq);
   const void *scales = g.scales;
   if constexpr (kGrouped) {
-    // blockIdx.y counts row tiles over all experts.  Every wave finds the expert on its own: lane l
-    // takes expert base+l, an inclusive scan over the lanes gives the running tile count, and the
-    // first lane whose count exceeds blockIdx.y owns the tile.
-    int t = blockIdx.y;
+    // Row tiles are counted over all experts.  Every wave works the numbering out on its own: lane l
+    // takes expert base+l and an inclusive scan over the lanes gives the running tile count.
+    // Workgroups are handed to the 8 XCDs in turn (linear id mod 8) and each XCD has its own L2, so
+    // the tiles are numbered expert by expert, row tile by row tile, column tile last, and XCD x
+    // takes the x-th contiguous eighth of that list: one expert's weights (and one row tile's
+    // activations) are then fetched into one L2 instead of all eight.  The grid is an upper bound
+    // padded to a multiple of 8; the exact number of tiles comes from the offsets.
+    const int64_t col_tiles = (C + BC - 1) / BC;
+    int total_rt = 0;
+    for (int base = 0; base < g.num_experts; base += 64) {
+      const int my = base + lane;
+      int tiles = 0;
+      if (my < g.num_experts) tiles = (g.offsets[my + 1] - g.offsets[my] + BM - 1) / BM;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) tiles += __shfl_xor(tiles, o, 64);
+      total_rt += tiles;
+    }
+    const int64_t total = static_cast<int64_t>(total_rt) * col_tiles;
+    const int64_t per_xcd = (total + 7) >> 3;
+    const int64_t slot = blockIdx.x >> 3;
+    const int64_t pos = static_cast<int64_t>(blockIdx.x & 7) * per_xcd + slot;
+    if (slot >= per_xcd || pos >= total) return;
+    int t = static_cast<int>(pos / col_tiles);
+    col_tile = pos - static_cast<int64_t>(t) * col_tiles;
     int e = 0;
     int64_t lo = 0, hi = 0;
     bool found = false;
@@ -584,7 +604,7 @@ int launch_one(const TileArgs &t, int64_t row_tiles, hipStream_t s)
   }
   const int64_t col_tiles = (C + BC - 1) / BC;
   dim3 grid(static_cast<unsigned>(col_tiles), static_cast<unsigned>(row_tiles));
-  if (!kGrouped) {
+  {
     const int64_t padded = (row_tiles * col_tiles + 7) / 8 * 8;      // linear grid, see the tile numbering in the kernel
     if (padded > 0x7fffffff) return CAIFX_ERR_UNSUPPORTED;
     grid = dim3(static_cast<unsigned>(padded), 1);
