@@ -61,9 +61,8 @@ def _check_segments(orc, rng, counts, N, K, kind, group=128):
 
 
 @pytest.mark.parametrize("kind", ["int8pc", "int4", "int8pt"])
-def test_grouped_long_segments_take_tall_tiles(orc, kind):
-    # a mean of more than 160 rows per expert switches the int8 kernels and the int4 input gradient
-    # to 256-row tiles: full tiles, a partial last tile, an empty expert
+def test_grouped_long_segments(orc, kind):
+    # segments of several tiles: full tiles, a partial last tile, an empty expert, a segment that ends on a tile edge
     _check_segments(orc, np.random.default_rng(11), np.array([300, 0, 517, 256]), 192, 256, kind)
 
 
