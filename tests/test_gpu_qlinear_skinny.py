@@ -69,6 +69,17 @@ def test_ragged_and_wave_count_variants(orc, N, K, M):
     _check(orc, rng, M, N, K, "int8pc", 2, 2)
 
 
+@pytest.mark.parametrize("N,K", [(4097, 4096), (2049, 2048), (1793, 4096), (6145, 1024), (8193, 4096)])
+@pytest.mark.parametrize("M", [1, 2])
+def test_row_streaming_tails(orc, N, K, M):
+    # one and two activation rows stream whole weight rows through a small ring per wave; these row
+    # counts leave a last wave with a single row (fewer rows than the ring holds), waves with no rows
+    # at all inside the last workgroup, and residue classes of unequal size for the per-channel scales
+    rng = np.random.default_rng(N + K + M)
+    for kind in ("int4", "int8pc", "int8pt"):
+        _check(orc, rng, M, N, K, kind, 2, 2)
+
+
 @pytest.mark.parametrize("N,K,M", [(1536, 1024, 6), (14336, 4096, 4), (200, 4096, 3), (2050, 640, 11)])
 def test_residue_classes_and_masked_row_blocks(orc, N, K, M):
     # 3 <= M <= 16 runs on the matrix cores in blocks of 16 weight rows: N = 200 and 2050 leave a
