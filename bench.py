@@ -278,8 +278,7 @@ def moe_rows(torch, T, dev, gen):
 
     def bwd():
         T.qlinear_grouped_backward_input(gout, offsets, down, T.BF16, T.BF16, out=gh, workspace=ws)
-        grad_up = T.multiply(gh, T.silu(gate_o))
-        grad_gate = T.silu_backward(gate_o, T.multiply(gh, up_o))
+        grad_gate, grad_up = T.swiglu_backward(gate_o, up_o, gh)
         T.qlinear_grouped_backward_input(grad_up, offsets, up, T.BF16, T.BF16, out=gi_up, workspace=ws)
         T.qlinear_grouped_backward_input(grad_gate, offsets, gate, T.BF16, T.BF16, out=gi_gate, workspace=ws)
         state["dx"] = T.add(gi_up, gi_gate)
@@ -339,6 +338,10 @@ def moe_rows(torch, T, dev, gen):
             "grouped_gemm_TFLOPs_fwd": round(gemm_flops / (ms_f * 1e-3) / 1e12, 1),
             "grouped_gemm_TFLOPs_bwd": round(gemm_flops / (ms_b * 1e-3) / 1e12, 1),
             "grouped_frac_of_mfma_peak": round(2 * gemm_flops / ((ms_f + ms_b) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+            # the other bound of a pass: every expert weight (int8 codes + fp32 per-channel scales) streamed once
+            "weight_bytes_per_pass": int(3 * E * D * H + E * (2 * H + D) * 4),
+            "weight_stream_us_at_hbm_peak": round((3 * E * D * H + E * (2 * H + D) * 4) / (HBM_PEAK_GBS * 1e9) * 1e6, 1),
+            "mfma_us_at_peak_per_pass": round(gemm_flops / (MFMA_BF16_PEAK_TFLOPS * 1e12) * 1e6, 1),
             "single_segment_replay_gate_proj": segments}
 
 

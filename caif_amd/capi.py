@@ -27,6 +27,7 @@ EXPORTS = [
     "caifx_qlinear_grouped_forward", "caifx_qlinear_grouped_backward_input",
     "caifx_qlinear_grouped_workspace_bytes",
     "caifx_silu", "caifx_silu_backward", "caifx_multiply", "caifx_add", "caifx_silu_multiply",
+    "caifx_swiglu_backward",
     "caifx_moe_dispatch_map_workspace_bytes", "caifx_moe_build_dispatch_map", "caifx_moe_dispatch",
     "caifx_moe_combine", "caifx_moe_combine_backward_grad_expert", "caifx_moe_combine_backward_grad_weights",
     "caifx_moe_dispatch_backward",
@@ -86,6 +87,7 @@ def lib():
         L.caifx_multiply.argtypes = [_p, _p, _p, _i64, _int, _p]
         L.caifx_add.argtypes = [_p, _p, _p, _i64, _int, _p]
         L.caifx_silu_multiply.argtypes = [_p, _p, _p, _i64, _int, _p]
+        L.caifx_swiglu_backward.argtypes = [_p, _p, _p, _p, _p, _i64, _int, _p]
         L.caifx_moe_dispatch_map_workspace_bytes.restype = _sz
         L.caifx_moe_dispatch_map_workspace_bytes.argtypes = [_i64, _int, _int]
         L.caifx_moe_build_dispatch_map.argtypes = [_p, _i64, _int, _int, _int, _p, _p, _p, _sz, _p]

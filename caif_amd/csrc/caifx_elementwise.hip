@@ -66,6 +66,55 @@ int launch_ew(const void *a, const void *b, void *out, int64_t n, hipStream_t s,
   return launch_status();
 }
 
+// Backward of hidden = silu(gate) * up as the reference chains four kernels, with every intermediate
+// rounded to T exactly where those kernels round:
+//   act = T(silu(gate));  grad_up = T(grad_hidden * act);
+//   t = T(grad_hidden * up);  grad_gate = T(silu'(gate) applied to t)
+// Three tensors in, two out, one pass.
+template <typename T>
+__global__ void swiglu_bwd_kernel(const T *__restrict__ gate, const T *__restrict__ up, const T *__restrict__ gh,
+                                  T *__restrict__ grad_gate, T *__restrict__ grad_up, int64_t n, int64_t n_body)
+{
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  auto one = [&](T g16, T u16, T h16, T &gg, T &gu) {
+    const float g = to_f32<T>(g16), u = to_f32<T>(u16), h = to_f32<T>(h16);
+    const float act = round_through<T>(SiluOp{}(g, 0.0f));
+    gu = from_f32<T>(MulOp{}(h, act));
+    const float tt = round_through<T>(MulOp{}(h, u));
+    gg = from_f32<T>(SiluBwdOp{}(g, tt));
+  };
+  const int64_t i = t * kVec;
+  if (i < n_body) {
+    T vg[kVec], vu[kVec], vh[kVec], og[kVec], ou[kVec];
+#pragma unroll
+    for (int j = 0; j < kVec; ++j) vg[j] = gate[i + j];
+#pragma unroll
+    for (int j = 0; j < kVec; ++j) vu[j] = up[i + j];
+#pragma unroll
+    for (int j = 0; j < kVec; ++j) vh[j] = gh[i + j];
+#pragma unroll
+    for (int j = 0; j < kVec; ++j) one(vg[j], vu[j], vh[j], og[j], ou[j]);
+#pragma unroll
+    for (int j = 0; j < kVec; ++j) grad_gate[i + j] = og[j];
+#pragma unroll
+    for (int j = 0; j < kVec; ++j) grad_up[i + j] = ou[j];
+  } else {
+    const int64_t k = n_body + (t - n_body / kVec);
+    if (k < n) one(gate[k], up[k], gh[k], grad_gate[k], grad_up[k]);
+  }
+}
+
+template <typename T>
+int launch_swiglu_bwd(const void *gate, const void *up, const void *gh, void *grad_gate, void *grad_up, int64_t n, hipStream_t s)
+{
+  const int64_t n_body = (n / kVec) * kVec;
+  const int64_t threads = n_body / kVec + (n - n_body);
+  hipLaunchKernelGGL((swiglu_bwd_kernel<T>), dim3(static_cast<unsigned>((threads + kBlock - 1) / kBlock)), dim3(kBlock), 0, s,
+                     static_cast<const T *>(gate), static_cast<const T *>(up), static_cast<const T *>(gh),
+                     static_cast<T *>(grad_gate), static_cast<T *>(grad_up), n, n_body);
+  return launch_status();
+}
+
 template <typename Op, bool kBinary>
 int dispatch_ew(const void *a, const void *b, void *out, int64_t n, int dtype, caifx_stream_t stream, Op op)
 {
@@ -114,6 +163,20 @@ int caifx_silu_multiply(const void *gate, const void *up, void *hidden, int64_t 
     case CAIFX_F32: return launch_ew<float, SiluMulOp<float>, true>(gate, up, hidden, n, s, SiluMulOp<float>{});
     case CAIFX_F16: return launch_ew<f16_t, SiluMulOp<f16_t>, true>(gate, up, hidden, n, s, SiluMulOp<f16_t>{});
     case CAIFX_BF16: return launch_ew<bf16_t, SiluMulOp<bf16_t>, true>(gate, up, hidden, n, s, SiluMulOp<bf16_t>{});
+    default: return CAIFX_ERR_INVALID_ARGUMENT;
+  }
+}
+
+int caifx_swiglu_backward(const void *gate, const void *up, const void *grad_hidden, void *grad_gate, void *grad_up,
+                          int64_t n, int dtype, caifx_stream_t stream)
+{
+  if (n <= 0) return CAIFX_OK;
+  if (!gate || !up || !grad_hidden || !grad_gate || !grad_up) return CAIFX_ERR_INVALID_ARGUMENT;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case CAIFX_F32: return launch_swiglu_bwd<float>(gate, up, grad_hidden, grad_gate, grad_up, n, s);
+    case CAIFX_F16: return launch_swiglu_bwd<f16_t>(gate, up, grad_hidden, grad_gate, grad_up, n, s);
+    case CAIFX_BF16: return launch_swiglu_bwd<bf16_t>(gate, up, grad_hidden, grad_gate, grad_up, n, s);
     default: return CAIFX_ERR_INVALID_ARGUMENT;
   }
 }

@@ -147,14 +147,11 @@ class CAIF_DeviceMoEFrozenExpert:public CAIF_DeviceLayerTyped<ComputeT,StorageT>
           CAIF_Ops::SiLUBackward(_cached_up_out,grad_hidden,grad_up);
           return AsStorage(Layer(_sub.up)->Backward(grad_up,ctx));
         }
-        CAIF_DeviceTensor gate_act=CAIF_DeviceTensor::Uninitialized(hshape,Stream(),sd);
-        CAIF_Ops::SiLU(_cached_gate_out,gate_act);
+        // grad_up = grad_hidden * silu(gate_out); grad_gate = SiLUBackward(gate_out, grad_hidden * up_out):
+        // the reference's four launches in one, same bits
         CAIF_DeviceTensor grad_up=CAIF_DeviceTensor::Uninitialized(hshape,Stream(),sd);
-        CAIF_Ops::Multiply(grad_hidden,gate_act,grad_up);
-        CAIF_DeviceTensor grad_gate_act=CAIF_DeviceTensor::Uninitialized(hshape,Stream(),sd);
-        CAIF_Ops::Multiply(grad_hidden,_cached_up_out,grad_gate_act);
         CAIF_DeviceTensor grad_gate=CAIF_DeviceTensor::Uninitialized(hshape,Stream(),sd);
-        CAIF_Ops::SiLUBackward(_cached_gate_out,grad_gate_act,grad_gate);
+        CAIF_Ops::SwiGLUBackward(_cached_gate_out,_cached_up_out,grad_hidden,grad_gate,grad_up);
         CAIF_DeviceTensor gi_up=AsStorage(Layer(_sub.up)->Backward(grad_up,ctx));
         CAIF_DeviceTensor gi_gate=AsStorage(Layer(_sub.gate)->Backward(grad_gate,ctx));
         CAIF_DeviceTensor grad_input=CAIF_DeviceTensor::Uninitialized({tokens,_config.InputDim()},Stream(),sd);

@@ -188,6 +188,24 @@ class CAIF_Ops
       }
       CAIF_CATCH_BLOCK()
     }
+    // SiLU, Multiply, Multiply, SiLUBackward of the gated expert's backward pass in one launch; the bits equal
+    // the four-op chain (every intermediate is rounded where those ops round)
+    static void SwiGLUBackward(const CAIF_DeviceTensor &gate,const CAIF_DeviceTensor &up,const CAIF_DeviceTensor &grad_hidden,
+                               CAIF_DeviceTensor &grad_gate,CAIF_DeviceTensor &grad_up)
+    {
+      try
+      {
+        SameKind(gate,up,"SwiGLUBackward");
+        SameKind(gate,grad_hidden,"SwiGLUBackward");
+        SameKind(gate,grad_gate,"SwiGLUBackward");
+        SameKind(gate,grad_up,"SwiGLUBackward");
+        Check(caifx_swiglu_backward(gate.DeviceDataRaw(),up.DeviceDataRaw(),grad_hidden.DeviceDataRaw(),
+                                    grad_gate.DeviceDataRaw(),grad_up.DeviceDataRaw(),
+                                    static_cast<int64_t>(gate.TotalElements()),CAIF_DataType(gate.Dtype()).CaifxCode(),
+                                    grad_gate.StreamHandle()),"SwiGLUBackward");
+      }
+      CAIF_CATCH_BLOCK()
+    }
     static void Multiply(const CAIF_DeviceTensor &a,const CAIF_DeviceTensor &b,CAIF_DeviceTensor &output)
     {
       try

@@ -227,6 +227,18 @@ def silu_multiply(gate, up):
     return _ew("caifx_silu_multiply", 2, gate, up)
 
 
+def swiglu_backward(gate, up, grad_hidden, out_gate=None, out_up=None):
+    """(grad_gate, grad_up) of hidden = silu(gate) * up in one pass, bit-identical to
+    multiply(grad_hidden, silu(gate)) and silu_backward(gate, multiply(grad_hidden, up))."""
+    _need_cuda(gate, up, grad_hidden)
+    assert gate.shape == up.shape == grad_hidden.shape and gate.dtype == up.dtype == grad_hidden.dtype
+    grad_gate = torch.empty_like(gate) if out_gate is None else out_gate
+    grad_up = torch.empty_like(gate) if out_up is None else out_up
+    capi.call("caifx_swiglu_backward", _ptr(gate), _ptr(up), _ptr(grad_hidden), _ptr(grad_gate), _ptr(grad_up),
+              gate.numel(), CODE_OF[gate.dtype], _stream())
+    return grad_gate, grad_up
+
+
 # ------------------------------------------------------------------ MoE token routing
 def moe_build_dispatch_map(expert_indices, num_experts, capacity_per_expert=0):
     """(dispatch_map [T, top_k] int32, expert_offsets [E+1] int32), built on the device without a host

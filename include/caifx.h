@@ -196,6 +196,14 @@ CAIFX_API int caifx_add(const void *a, const void *b, void *output, int64_t n, i
  * The intermediate rounding of silu(gate) to T is kept, so the bits equal the two-op sequence. */
 CAIFX_API int caifx_silu_multiply(const void *gate, const void *up, void *hidden, int64_t n, int dtype,
                         caifx_stream_t stream);
+/* The element-wise part of CAIF_DeviceMoEFrozenExpert::BackwardImpl for the gated expert
+ * (src/caif_device_moe_frozen_expert.cpp:266-289: SiLU, Multiply, Multiply, SiLUBackward) in one pass:
+ *   grad_up   = T(float(grad_hidden) * float(T(silu(gate))))
+ *   grad_gate = T(silu_backward(gate, T(float(grad_hidden) * float(up))))
+ * Every intermediate is rounded to T where the four kernels round, so the bits equal the four-op
+ * sequence.  The outputs must not alias the inputs. */
+CAIFX_API int caifx_swiglu_backward(const void *gate, const void *up, const void *grad_hidden, void *grad_gate,
+                          void *grad_up, int64_t n, int dtype, caifx_stream_t stream);
 
 /* ---------------------------------------------------------------------------
  * MoE token routing around the grouped dequant-GEMMs: the dispatch map, the gather into the

@@ -159,3 +159,27 @@ def test_elementwise_ops_match_oracle(orc):
             assert np.all(np.abs(g - w) <= ulp * np.maximum(np.abs(w), 1e-3) * 1.01)
         assert np.array_equal(host(T.multiply(ad, bd)), orc.multiply(ah, bh, dt))   # exact
         assert np.array_equal(host(T.add(ad, bd)), orc.add(ah, bh, dt))             # exact
+
+
+def test_fused_swiglu_backward_equals_the_four_op_chain(orc):
+    # grad_up = grad_hidden * silu(gate), grad_gate = silu_backward(gate, grad_hidden * up): the fused kernel rounds
+    # every intermediate where the four kernels round, so the bits are those of the chain (same device expf),
+    # and the oracle's chain agrees to one ulp of the tensor dtype (libm's expf differs by a few ulp)
+    rng = np.random.default_rng(40)
+    n = 8 * 1234 + 3                                                 # vector body + scalar tail
+    g = rng.normal(0, 2, n).astype(np.float32)
+    u = rng.normal(0, 2, n).astype(np.float32)
+    h = rng.normal(0, 1, n).astype(np.float32)
+    for dt in (0, 2, 1):
+        gd, ud, hd = dev_as(g, dt), dev_as(u, dt), dev_as(h, dt)
+        gg, gu = T.swiglu_backward(gd, ud, hd)
+        want_gu = T.multiply(hd, T.silu(gd))
+        want_gg = T.silu_backward(gd, T.multiply(hd, ud))
+        assert np.array_equal(host(gu), host(want_gu)), dt
+        assert np.array_equal(host(gg), host(want_gg)), dt
+        gh_, uh_, hh_ = host(gd), host(ud), host(hd)
+        ulp = {0: 2e-6, 1: 2 ** -10, 2: 2 ** -7}[dt]
+        o_gu = orc.multiply(hh_, orc.silu(gh_, dt), dt)
+        o_gg = orc.silu_backward(gh_, orc.multiply(hh_, uh_, dt), dt)
+        assert np.all(np.abs(host(gu) - o_gu) <= ulp * np.maximum(np.abs(o_gu), 1e-3) * 1.01)
+        assert np.all(np.abs(host(gg) - o_gg) <= 2 * ulp * np.maximum(np.abs(o_gg), 1e-3) * 1.01)
