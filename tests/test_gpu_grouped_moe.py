@@ -66,6 +66,33 @@ def test_grouped_long_segments(orc, kind):
     _check_segments(orc, np.random.default_rng(11), np.array([300, 0, 517, 256]), 192, 256, kind)
 
 
+def test_grouped_full_size_config5_sampled_experts(orc):
+    # BASELINE configs[4] geometry: 64 experts, 4096 tokens x top-6 = 24576 packed rows, gate/up projection
+    # 2048 -> 1408 with int8 per-channel weights.  The oracle checks three sampled experts (first, a middle
+    # one, last); a size-independent property covers all of them: doubling the activations doubles every
+    # output row exactly (power-of-two scaling commutes with every rounding on the path).
+    rng = np.random.default_rng(64)
+    E, N, K, tokens, top_k = 64, 1408, 2048, 4096, 6
+    counts = np.bincount(rng.integers(0, E, tokens * top_k), minlength=E)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    total = int(offsets[-1])
+    ows, gw = _experts(orc, rng, E, N, K, "int8pc")
+    x = dev_as(rng.normal(0, 1, (total, K)), 2)
+    dy = dev_as(rng.normal(0, 1e-2, (total, N)), 2)
+    off_d = dev(offsets)
+    y = T.qlinear_grouped_forward(x, off_d, gw, 2)
+    dx = T.qlinear_grouped_backward_input(dy, off_d, gw, 2)
+    y2 = T.qlinear_grouped_forward(x * 2, off_d, gw, 2)
+    dx2 = T.qlinear_grouped_backward_input(dy * 2, off_d, gw, 2)
+    assert torch.equal(y2, y * 2) and torch.equal(dx2, dx * 2)
+    yh, dxh, xh, dyh = host(y), host(dx), host(x), host(dy)
+    for e in (0, 31, 63):
+        lo, hi = offsets[e], offsets[e + 1]
+        assert hi > lo
+        assert max_rel_err(yh[lo:hi], orc.frozen_linear_forward(xh[lo:hi], ows[e], 2)) <= 5e-5, e
+        assert max_rel_err(dxh[lo:hi], orc.frozen_linear_backward(dyh[lo:hi], ows[e], 2)) <= 5e-5, e
+
+
 def test_grouped_more_experts_than_lanes(orc):
     # 70 experts: the tile -> expert search runs over more than one 64-lane chunk of the offsets
     rng = np.random.default_rng(12)

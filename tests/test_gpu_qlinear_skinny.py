@@ -80,7 +80,7 @@ def test_row_streaming_tails(orc, N, K, M):
         _check(orc, rng, M, N, K, kind, 2, 2)
 
 
-@pytest.mark.parametrize("N,K,M", [(1536, 1024, 6), (14336, 4096, 4), (200, 4096, 3), (2050, 640, 11)])
+@pytest.mark.parametrize("N,K,M", [(1536, 1024, 6), (14336, 4096, 4), (14336, 4096, 16), (200, 4096, 3), (2050, 640, 11)])
 def test_residue_classes_and_masked_row_blocks(orc, N, K, M):
     # 3 <= M <= 16 runs on the matrix cores in blocks of 16 weight rows: N = 200 and 2050 leave a
     # partly masked last block; int8 per-channel scales (period N) split the rows into
