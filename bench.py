@@ -240,6 +240,33 @@ def compute_bound_rows(torch, T, dev, gen, capture, time_graph):
             rows[key].update({"dx_us": round(ms_b * 1e3, 2), "dx_TFLOPs": round(flops / (ms_b * 1e-3) / 1e12, 1),
                               "fwd_dx_frac_of_mfma_peak":
                                   round(2 * flops / ((ms_f + ms_b) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+        if (M, N) == (4096, 11008):
+            # configs[3]: what the LoRA adapter does with the frozen base around its own small GEMMs: the base
+            # output cast to bf16 and added to the low-rank branch, forward and backward.  "chain" is the
+            # reference's sequence (fp32 result, cast, Add); "fused" folds cast and Add into the GEMM's store.
+            lora_y = torch.empty(M, N, device=dev).normal_(0, 1e-2, generator=gen).to(torch.bfloat16)
+            lora_x = torch.empty(M, K, device=dev).normal_(0, 1e-4, generator=gen).to(torch.bfloat16)
+            yb = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+            xb = torch.empty(M, K, device=dev, dtype=torch.bfloat16)
+
+            def chain(i):
+                T.qlinear_forward(x, fw, T.BF16, T.F32, out=y, workspace=ws)
+                T.add(y.to(torch.bfloat16), lora_y)
+                T.qlinear_backward_input(dy, fw, T.BF16, T.F32, out=dx, workspace=ws)
+                T.add(dx.to(torch.bfloat16), lora_x)
+
+            def fused(i):
+                T.qlinear_forward(x, fw, T.BF16, T.BF16, out=yb, workspace=ws, addend=lora_y)
+                T.qlinear_backward_input(dy, fw, T.BF16, T.BF16, out=xb, workspace=ws, addend=lora_x)
+
+            g = capture(chain, 4)
+            ms_c = time_graph(g, 4, reps=3)
+            del g
+            g = capture(fused, 4)
+            ms_u = time_graph(g, 4, reps=3)
+            del g
+            rows["lora_base_fwd_bwd_M4096_N11008_K4096"] = {
+                "gemm_cast_add_chain_us": round(ms_c * 1e3, 1), "fused_store_us": round(ms_u * 1e3, 1)}
     return {"prefill_gemm": rows, "moe_frozen_experts": moe_rows(torch, T, dev, gen)}
 
 
@@ -280,8 +307,9 @@ def moe_rows(torch, T, dev, gen):
         T.qlinear_grouped_backward_input(gout, offsets, down, T.BF16, T.BF16, out=gh, workspace=ws)
         grad_gate, grad_up = T.swiglu_backward(gate_o, up_o, gh)
         T.qlinear_grouped_backward_input(grad_up, offsets, up, T.BF16, T.BF16, out=gi_up, workspace=ws)
-        T.qlinear_grouped_backward_input(grad_gate, offsets, gate, T.BF16, T.BF16, out=gi_gate, workspace=ws)
-        state["dx"] = T.add(gi_up, gi_gate)
+        # gi_up + gi_gate folded into the second GEMM's store (same bits as the reference's Add)
+        state["dx"] = T.qlinear_grouped_backward_input(grad_gate, offsets, gate, T.BF16, T.BF16, out=gi_gate,
+                                                       workspace=ws, addend=gi_up)
 
     def timed(fn, iters=10):
         fn()

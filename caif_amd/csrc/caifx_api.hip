@@ -88,38 +88,86 @@ size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtyp
   return mfma_workspace_bytes(a, backward != 0);
 }
 
-int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K, const void *x, int x_dtype, int compute_dtype,
-                          const void *wq, int w_kind, const void *scales, int64_t scale_period, int group_size,
-                          void *y, int y_dtype, void *workspace, size_t workspace_bytes, caifx_stream_t stream)
+// `addend` (optional): the matrix-core GEMM adds it in its store; every other path runs as usual and is
+// followed by the element-wise Add in place, which rounds in the same two places
+static int finish_add(int st, const void *addend, void *y, int y_dtype, int64_t n, caifx_stream_t stream)
+{
+  if (st != CAIFX_OK || !addend) return st;
+  return caifx_add(y, addend, y, n, y_dtype, stream);
+}
+
+static int forward_impl(int64_t M, int64_t N, int64_t K, const void *x, int x_dtype, int compute_dtype,
+                        const void *wq, int w_kind, const void *scales, int64_t scale_period, int group_size,
+                        void *y, int y_dtype, const void *addend, void *workspace, size_t workspace_bytes,
+                        caifx_stream_t stream)
 {
   int st = validate_common(M, N, K, x, x_dtype, compute_dtype, y, y_dtype);
   if (st != CAIFX_OK) return st;
   if (!wq) return CAIFX_ERR_INVALID_ARGUMENT;
   st = validate_weight(N, K, w_kind, scales, scale_period, group_size);
   if (st != CAIFX_OK) return st;
+  if (addend && (addend == y || !aligned_to(addend, dtype_size(y_dtype)))) return CAIFX_ERR_INVALID_ARGUMENT;
   if (M == 0) return CAIFX_OK;
-  const GemmArgs a = make_args(M, N, K, x, x_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, y,
-                               y_dtype, workspace, workspace_bytes);
+  GemmArgs a = make_args(M, N, K, x, x_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, y,
+                         y_dtype, workspace, workspace_bytes);
   hipStream_t s = as_stream(stream);
   // one or two rows: stream each weight row linearly and reduce per row; from three rows on the
   // matrix-core tiling (cost independent of M) is faster; both fall through when a shape does not fit
-  if (M <= 2) {
-    st = rowlin_forward(a, s);
-    if (st != CAIFX_ERR_UNSUPPORTED) return st;
-  }
-  if (M <= 16) {
+  st = CAIFX_ERR_UNSUPPORTED;
+  if (M <= 2) st = rowlin_forward(a, s);
+  if (st == CAIFX_ERR_UNSUPPORTED && M <= 16) {
     st = mblock_forward(a, s);
-    if (st != CAIFX_ERR_UNSUPPORTED) return st;
-    if (M <= 4) {
-      st = rowlin_forward(a, s);
-      if (st != CAIFX_ERR_UNSUPPORTED) return st;
-    }
-    st = skinny_forward(a, s);
-    if (st != CAIFX_ERR_UNSUPPORTED) return st;
+    if (st == CAIFX_ERR_UNSUPPORTED && M <= 4) st = rowlin_forward(a, s);
+    if (st == CAIFX_ERR_UNSUPPORTED) st = skinny_forward(a, s);
   }
-  st = mfma_forward(a, s);
-  if (st != CAIFX_ERR_UNSUPPORTED) return st;
-  return generic_forward(a, s);
+  if (st == CAIFX_ERR_UNSUPPORTED) {
+    a.addend = addend;
+    st = mfma_forward(a, s);
+    if (st != CAIFX_ERR_UNSUPPORTED) return st;       // added in the store
+    a.addend = nullptr;
+    st = generic_forward(a, s);
+  }
+  return finish_add(st, addend, y, y_dtype, M * N, stream);
+}
+
+int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K, const void *x, int x_dtype, int compute_dtype,
+                          const void *wq, int w_kind, const void *scales, int64_t scale_period, int group_size,
+                          void *y, int y_dtype, void *workspace, size_t workspace_bytes, caifx_stream_t stream)
+{
+  return forward_impl(M, N, K, x, x_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, y, y_dtype,
+                      nullptr, workspace, workspace_bytes, stream);
+}
+
+int caifx_qlinear_forward_add(int64_t M, int64_t N, int64_t K, const void *x, int x_dtype, int compute_dtype,
+                              const void *wq, int w_kind, const void *scales, int64_t scale_period, int group_size,
+                              void *y, int y_dtype, const void *addend, void *workspace, size_t workspace_bytes,
+                              caifx_stream_t stream)
+{
+  if (M > 0 && !addend) return CAIFX_ERR_INVALID_ARGUMENT;
+  return forward_impl(M, N, K, x, x_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, y, y_dtype,
+                      addend, workspace, workspace_bytes, stream);
+}
+
+static int backward_impl(int64_t M, int64_t N, int64_t K, const void *dy, int dy_dtype, int compute_dtype,
+                         const void *wq, int w_kind, const void *scales, int64_t scale_period, int group_size,
+                         void *dx, int dx_dtype, const void *addend, void *workspace, size_t workspace_bytes,
+                         caifx_stream_t stream)
+{
+  int st = validate_common(M, N, K, dy, dy_dtype, compute_dtype, dx, dx_dtype);
+  if (st != CAIFX_OK) return st;
+  if (!wq) return CAIFX_ERR_INVALID_ARGUMENT;
+  st = validate_weight(N, K, w_kind, scales, scale_period, group_size);
+  if (st != CAIFX_OK) return st;
+  if (addend && (addend == dx || !aligned_to(addend, dtype_size(dx_dtype)))) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (M == 0) return CAIFX_OK;
+  GemmArgs a = make_args(M, N, K, dy, dy_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size,
+                         dx, dx_dtype, workspace, workspace_bytes);
+  hipStream_t s = as_stream(stream);
+  a.addend = addend;
+  st = mfma_backward(a, s);
+  if (st != CAIFX_ERR_UNSUPPORTED) return st;         // added in the store
+  a.addend = nullptr;
+  return finish_add(generic_backward(a, s), addend, dx, dx_dtype, M * K, stream);
 }
 
 int caifx_qlinear_backward_input(int64_t M, int64_t N, int64_t K, const void *dy, int dy_dtype, int compute_dtype,
@@ -127,18 +175,18 @@ int caifx_qlinear_backward_input(int64_t M, int64_t N, int64_t K, const void *dy
                                  int group_size, void *dx, int dx_dtype, void *workspace, size_t workspace_bytes,
                                  caifx_stream_t stream)
 {
-  int st = validate_common(M, N, K, dy, dy_dtype, compute_dtype, dx, dx_dtype);
-  if (st != CAIFX_OK) return st;
-  if (!wq) return CAIFX_ERR_INVALID_ARGUMENT;
-  st = validate_weight(N, K, w_kind, scales, scale_period, group_size);
-  if (st != CAIFX_OK) return st;
-  if (M == 0) return CAIFX_OK;
-  const GemmArgs a = make_args(M, N, K, dy, dy_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size,
-                               dx, dx_dtype, workspace, workspace_bytes);
-  hipStream_t s = as_stream(stream);
-  st = mfma_backward(a, s);
-  if (st != CAIFX_ERR_UNSUPPORTED) return st;
-  return generic_backward(a, s);
+  return backward_impl(M, N, K, dy, dy_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, dx,
+                       dx_dtype, nullptr, workspace, workspace_bytes, stream);
+}
+
+int caifx_qlinear_backward_input_add(int64_t M, int64_t N, int64_t K, const void *dy, int dy_dtype, int compute_dtype,
+                                     const void *wq, int w_kind, const void *scales, int64_t scale_period,
+                                     int group_size, void *dx, int dx_dtype, const void *addend, void *workspace,
+                                     size_t workspace_bytes, caifx_stream_t stream)
+{
+  if (M > 0 && !addend) return CAIFX_ERR_INVALID_ARGUMENT;
+  return backward_impl(M, N, K, dy, dy_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, dx,
+                       dx_dtype, addend, workspace, workspace_bytes, stream);
 }
 
 size_t caifx_qlinear_grouped_workspace_bytes(int num_experts, int64_t total_rows, int64_t N, int64_t K, int x_dtype,
@@ -159,7 +207,7 @@ size_t caifx_qlinear_grouped_workspace_bytes(int num_experts, int64_t total_rows
 static int grouped(bool backward, int num_experts, const int32_t *offsets, int64_t total_rows, int64_t N, int64_t K,
                    const void *x, int x_dtype, int compute_dtype, const void *const *wq_ptrs, int w_kind,
                    const void *const *scales_ptrs, int64_t scale_period, int group_size, void *y, int y_dtype,
-                   void *workspace, size_t workspace_bytes, caifx_stream_t stream)
+                   const void *addend, void *workspace, size_t workspace_bytes, caifx_stream_t stream)
 {
   int st = validate_common(total_rows, N, K, x, x_dtype, compute_dtype, y, y_dtype);
   if (st != CAIFX_OK) return st;
@@ -180,9 +228,14 @@ static int grouped(bool backward, int num_experts, const int32_t *offsets, int64
   a.wq_ptrs = wq_ptrs;
   a.scales_ptrs = scales_ptrs;
   a.num_experts = num_experts;
+  if (addend && (addend == y || !aligned_to(addend, dtype_size(y_dtype)))) return CAIFX_ERR_INVALID_ARGUMENT;
   hipStream_t s = as_stream(stream);
+  a.addend = addend;
   st = backward ? mfma_backward(a, s) : mfma_forward(a, s);
   if (st != CAIFX_ERR_UNSUPPORTED) return st;
+  // the shape-agnostic kernels have no fused add, and rows past offsets[E] must stay untouched, which a
+  // plain element-wise pass over the buffer would not respect
+  if (addend) return CAIFX_ERR_UNSUPPORTED;
   return backward ? generic_backward(a, s) : generic_forward(a, s);
 }
 
@@ -193,7 +246,7 @@ int caifx_qlinear_grouped_forward(int num_experts, const int32_t *offsets, int64
                                   caifx_stream_t stream)
 {
   return grouped(false, num_experts, offsets, total_rows, N, K, x, x_dtype, compute_dtype, wq_ptrs, w_kind,
-                 scales_ptrs, scale_period, group_size, y, y_dtype, workspace, workspace_bytes, stream);
+                 scales_ptrs, scale_period, group_size, y, y_dtype, nullptr, workspace, workspace_bytes, stream);
 }
 
 int caifx_qlinear_grouped_backward_input(int num_experts, const int32_t *offsets, int64_t total_rows, int64_t N,
@@ -203,7 +256,19 @@ int caifx_qlinear_grouped_backward_input(int num_experts, const int32_t *offsets
                                          void *workspace, size_t workspace_bytes, caifx_stream_t stream)
 {
   return grouped(true, num_experts, offsets, total_rows, N, K, dy, dy_dtype, compute_dtype, wq_ptrs, w_kind,
-                 scales_ptrs, scale_period, group_size, dx, dx_dtype, workspace, workspace_bytes, stream);
+                 scales_ptrs, scale_period, group_size, dx, dx_dtype, nullptr, workspace, workspace_bytes, stream);
+}
+
+int caifx_qlinear_grouped_backward_input_add(int num_experts, const int32_t *offsets, int64_t total_rows, int64_t N,
+                                             int64_t K, const void *dy, int dy_dtype, int compute_dtype,
+                                             const void *const *wq_ptrs, int w_kind, const void *const *scales_ptrs,
+                                             int64_t scale_period, int group_size, void *dx, int dx_dtype,
+                                             const void *addend, void *workspace, size_t workspace_bytes,
+                                             caifx_stream_t stream)
+{
+  if (total_rows > 0 && num_experts > 0 && !addend) return CAIFX_ERR_INVALID_ARGUMENT;
+  return grouped(true, num_experts, offsets, total_rows, N, K, dy, dy_dtype, compute_dtype, wq_ptrs, w_kind,
+                 scales_ptrs, scale_period, group_size, dx, dx_dtype, addend, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

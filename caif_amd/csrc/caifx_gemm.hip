@@ -58,6 +58,8 @@ struct TileArgs {
   const void *a;             // activations [M, R]
   void *d;                   // result [M, C]
   int d_dtype;
+  const void *addend;        // optional [M, C] of d_dtype: d = T(float(T(acc)) + float(addend))
+  int vec_store;             // 16-bit result, C % 8 == 0, 16-byte aligned pointers: the store goes through LDS in 16-byte pieces
   const void *wq;
   const void *scales;
   int group_shift;           // int4: log2(group_size)
@@ -560,6 +562,53 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
   }
 
   // ---- epilogue: acc[i][j][r] = D[row][col], row = 8*(r/4) + 4*(lane/32) + r%4, col = lane%32
+  // 16-bit results: a lane's values sit in 16 different rows, two bytes each, so a direct store moves 64-byte
+  // pieces.  After the last barrier nobody reads the operand tiles any more, so each consumer wave lays its
+  // (BM/2) x 64 sub-tile out in a private piece of LDS (row pitch 144 bytes: conflict free both ways) and
+  // writes it, and reads the optional addend, as 16 bytes per lane and 128 contiguous bytes per row.
+  if (g.vec_store) {
+    constexpr int kPitch = 64 * 2 + 16;
+    unsigned char *stage = smem + wave * (kWaveRows * kPitch);
+    auto staged = [&](auto tag) {
+      typedef decltype(tag) T;
+#pragma unroll
+      for (int i = 0; i < WR; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int lrow = i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            *reinterpret_cast<T *>(stage + lrow * kPitch + (j * 32 + (lane & 31)) * 2) = from_f32<T>(acc[i][j][r]);
+          }
+      // same wave, LDS executes a wave's accesses in order: only the compiler must not move the reads up
+      asm volatile("" ::: "memory");
+      const int chunk = lane & 7;
+      const int64_t gcol = col0 + wc * 64 + chunk * 8;
+#pragma unroll
+      for (int it = 0; it < kWaveRows / 8; ++it) {
+        const int lrow = it * 8 + (lane >> 3);
+        const int64_t grow = row_lo + wm * kWaveRows + lrow;
+        if (grow < row_hi && gcol < C) {
+          u32x4_t v = *reinterpret_cast<const u32x4_t *>(stage + lrow * kPitch + chunk * 16);
+          const int64_t o = grow * C + gcol;
+          if (g.addend) {
+            const u32x4_t av = *reinterpret_cast<const u32x4_t *>(static_cast<const T *>(g.addend) + o);
+            const T *vp = reinterpret_cast<const T *>(&v);
+            const T *ap = reinterpret_cast<const T *>(&av);
+            u32x4_t w;
+            T *wp = reinterpret_cast<T *>(&w);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) wp[e] = from_f32<T>(to_f32(vp[e]) + to_f32(ap[e]));
+            v = w;
+          }
+          *reinterpret_cast<u32x4_t *>(static_cast<T *>(g.d) + o) = v;
+        }
+      }
+    };
+    if (g.d_dtype == CAIFX_BF16) staged(bf16_t{});
+    else staged(f16_t{});
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < WR; ++i) {
 #pragma unroll
@@ -571,7 +620,13 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
           const int64_t row = row_lo + wm * kWaveRows + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
           if (row < row_hi) {
             const int64_t o = row * C + col;
-            const float v = acc[i][j][r];
+            float v = acc[i][j][r];
+            if (g.addend) {
+              // the caller's cast of this result to the tensor dtype followed by an element-wise Add, same roundings
+              if (g.d_dtype == CAIFX_F32) v += static_cast<const float *>(g.addend)[o];
+              else if (g.d_dtype == CAIFX_BF16) v = round_through<bf16_t>(v) + to_f32(static_cast<const bf16_t *>(g.addend)[o]);
+              else v = round_through<f16_t>(v) + to_f32(static_cast<const f16_t *>(g.addend)[o]);
+            }
             if (g.d_dtype == CAIFX_F32) static_cast<float *>(g.d)[o] = v;
             else if (g.d_dtype == CAIFX_BF16) static_cast<bf16_t *>(g.d)[o] = from_f32<bf16_t>(v);
             else static_cast<f16_t *>(g.d)[o] = from_f32<f16_t>(v);
@@ -683,6 +738,11 @@ int run(const GemmArgs &a, bool backward, hipStream_t s)
   t.a = a.x;
   t.d = a.y;
   t.d_dtype = a.y_dtype;
+  t.addend = a.addend;
+  {
+    const int64_t cols = backward ? a.K : a.N;
+    t.vec_store = a.y_dtype != CAIFX_F32 && cols % 8 == 0 && aligned_to(a.y, 16) && (!a.addend || aligned_to(a.addend, 16));
+  }
   t.wq = a.w.q;
   t.scales = a.w.scales;
   t.offsets = a.offsets;

@@ -29,6 +29,8 @@ struct GemmArgs {
   int num_experts;
   void *workspace;
   size_t workspace_bytes;
+  // optional: y = T(float(T(acc)) + float(addend)), addend [M, columns of y] of y_dtype (may alias y)
+  const void *addend;
 };
 
 int generic_forward(const GemmArgs &a, hipStream_t s);

@@ -271,20 +271,21 @@ class CAIF_DeviceMoEFrozenExpertBank
         const std::vector<uint32_t> hs={rows,_hidden_dim};
         CAIF_DeviceTensor grad_hidden=CAIF_DeviceTensor::Zeros(hs,*_stream,sd);
         Grouped(true,2,grad_out,offsets,grad_hidden,_input_dim,_hidden_dim);
-        CAIF_DeviceTensor gate_act=CAIF_DeviceTensor::Uninitialized(hs,*_stream,sd);
-        CAIF_Ops::SiLU(_gate_out,gate_act);
+        // the four element-wise launches of the gated backward in one, and gi_up + gi_gate folded into the second
+        // input-gradient GEMM's store: same bits as the reference's sequence
         CAIF_DeviceTensor grad_up=CAIF_DeviceTensor::Uninitialized(hs,*_stream,sd);
-        CAIF_Ops::Multiply(grad_hidden,gate_act,grad_up);
-        CAIF_DeviceTensor gga=CAIF_DeviceTensor::Uninitialized(hs,*_stream,sd);
-        CAIF_Ops::Multiply(grad_hidden,_up_out,gga);
         CAIF_DeviceTensor grad_gate=CAIF_DeviceTensor::Uninitialized(hs,*_stream,sd);
-        CAIF_Ops::SiLUBackward(_gate_out,gga,grad_gate);
+        CAIF_Ops::SwiGLUBackward(_gate_out,_up_out,grad_hidden,grad_gate,grad_up);
         CAIF_DeviceTensor gi_up=CAIF_DeviceTensor::Zeros({rows,_input_dim},*_stream,sd);
-        CAIF_DeviceTensor gi_gate=CAIF_DeviceTensor::Zeros({rows,_input_dim},*_stream,sd);
         Grouped(true,1,grad_up,offsets,gi_up,_hidden_dim,_input_dim);
-        Grouped(true,0,grad_gate,offsets,gi_gate,_hidden_dim,_input_dim);
-        CAIF_DeviceTensor grad_in=CAIF_DeviceTensor::Uninitialized({rows,_input_dim},*_stream,sd);
-        CAIF_Ops::Add(gi_up,gi_gate,grad_in);
+        CAIF_DeviceTensor grad_in=CAIF_DeviceTensor::Zeros({rows,_input_dim},*_stream,sd);
+        if(Grouped(true,0,grad_gate,offsets,grad_in,_hidden_dim,_input_dim,&gi_up)==false)
+        {
+          // shapes the matrix-core kernel does not take: plain call, then the Add
+          CAIF_DeviceTensor gi_gate=CAIF_DeviceTensor::Zeros({rows,_input_dim},*_stream,sd);
+          Grouped(true,0,grad_gate,offsets,gi_gate,_hidden_dim,_input_dim);
+          CAIF_Ops::Add(gi_up,gi_gate,grad_in);
+        }
         return grad_in;
       }
       CAIF_CATCH_BLOCK()
@@ -337,8 +338,10 @@ class CAIF_DeviceMoEFrozenExpertBank
       dev.CopyFromHostRaw(host.data(),host.size()*sizeof(void*));
     }
     // which: 0 gate, 1 up, 2 down.  N/K are the frozen linear's OutputDim/InputDim.
-    void Grouped(bool backward,int which,const CAIF_DeviceTensor &in,const CAIF_DeviceTensor &offsets,CAIF_DeviceTensor &out,
-                 uint32_t N,uint32_t K)
+    // addend (backward only): out = T(T(in * W_e) + addend) in the store; returns false when that form is not
+    // available for the shape (nothing has been launched then)
+    bool Grouped(bool backward,int which,const CAIF_DeviceTensor &in,const CAIF_DeviceTensor &offsets,CAIF_DeviceTensor &out,
+                 uint32_t N,uint32_t K,const CAIF_DeviceTensor *addend=nullptr)
     {
       const Kind_t &k=_kinds[which];
       const int code=CAIF_DataType(CAIF_DtypeOf<StorageT>::value).CaifxCode();
@@ -348,7 +351,17 @@ class CAIF_DeviceMoEFrozenExpertBank
       const int64_t rows=in.Shape()[0];
       const int32_t *off=static_cast<const int32_t*>(offsets.DeviceDataRaw());
       int st;
-      if(backward==true)
+      if(backward==true&&addend!=nullptr)
+      {
+        st=caifx_qlinear_grouped_backward_input_add(_num_experts,off,rows,N,K,in.DeviceDataRaw(),code,cc,wp,k.kind,sp,k.period,
+                                                    k.group,out.DeviceDataRaw(),code,addend->DeviceDataRaw(),nullptr,0,
+                                                    _stream->Handle());
+        if(st==CAIFX_ERR_UNSUPPORTED)
+        {
+          return false;
+        }
+      }
+      else if(backward==true)
       {
         st=caifx_qlinear_grouped_backward_input(_num_experts,off,rows,N,K,in.DeviceDataRaw(),code,cc,wp,k.kind,sp,k.period,
                                                 k.group,out.DeviceDataRaw(),code,nullptr,0,_stream->Handle());
@@ -359,6 +372,7 @@ class CAIF_DeviceMoEFrozenExpertBank
                                          out.DeviceDataRaw(),code,nullptr,0,_stream->Handle());
       }
       CAIF_Ops::Check(st,"MoEFrozenExpertBank: grouped dequant-GEMM");
+      return true;
     }
 
     CAIF_CudaStream *_stream;

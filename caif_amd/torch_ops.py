@@ -124,8 +124,9 @@ def _workspace(nbytes, device):
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
 
 
-def qlinear_forward(x, fw, compute_dtype, y_dtype=F32, out=None, workspace=None):
-    """caifx_qlinear_forward on x [..., K]; returns y [M, N]."""
+def qlinear_forward(x, fw, compute_dtype, y_dtype=F32, out=None, workspace=None, addend=None):
+    """caifx_qlinear_forward on x [..., K]; returns y [M, N].  With `addend` [M, N] of y_dtype:
+    caifx_qlinear_forward_add, y = T(float(T(x W^T)) + float(addend))."""
     _need_cuda(x)
     M = x.numel() // fw.K
     y = out if out is not None else torch.empty((M, fw.N), dtype=TORCH_DTYPE[y_dtype], device=x.device)
@@ -133,14 +134,20 @@ def qlinear_forward(x, fw, compute_dtype, y_dtype=F32, out=None, workspace=None)
     if workspace is None:
         workspace = _workspace(capi.lib().caifx_qlinear_workspace_bytes(M, fw.N, fw.K, xd, compute_dtype,
                                                                        fw.w_kind, 0), x.device)
+    if addend is not None:
+        assert addend.dtype == y.dtype and addend.numel() == y.numel()
+        capi.call("caifx_qlinear_forward_add", M, fw.N, fw.K, _ptr(x), xd, compute_dtype, _ptr(fw.wq), fw.w_kind,
+                  _ptr(fw.scales), fw.scale_period, fw.group_size, _ptr(y), y_dtype, _ptr(addend), _ptr(workspace),
+                  workspace.numel(), _stream())
+        return y
     capi.call("caifx_qlinear_forward", M, fw.N, fw.K, _ptr(x), xd, compute_dtype, _ptr(fw.wq), fw.w_kind,
               _ptr(fw.scales), fw.scale_period, fw.group_size, _ptr(y), y_dtype, _ptr(workspace),
               workspace.numel(), _stream())
     return y
 
 
-def qlinear_backward_input(dy, fw, compute_dtype, dx_dtype=F32, out=None, workspace=None):
-    """caifx_qlinear_backward_input on dy [..., N]; returns dx [M, K]."""
+def qlinear_backward_input(dy, fw, compute_dtype, dx_dtype=F32, out=None, workspace=None, addend=None):
+    """caifx_qlinear_backward_input on dy [..., N]; returns dx [M, K] (plus `addend` [M, K], see qlinear_forward)."""
     _need_cuda(dy)
     M = dy.numel() // fw.N
     dx = out if out is not None else torch.empty((M, fw.K), dtype=TORCH_DTYPE[dx_dtype], device=dy.device)
@@ -148,6 +155,12 @@ def qlinear_backward_input(dy, fw, compute_dtype, dx_dtype=F32, out=None, worksp
     if workspace is None:
         workspace = _workspace(capi.lib().caifx_qlinear_workspace_bytes(M, fw.N, fw.K, yd, compute_dtype,
                                                                        fw.w_kind, 1), dy.device)
+    if addend is not None:
+        assert addend.dtype == dx.dtype and addend.numel() == dx.numel()
+        capi.call("caifx_qlinear_backward_input_add", M, fw.N, fw.K, _ptr(dy), yd, compute_dtype, _ptr(fw.wq),
+                  fw.w_kind, _ptr(fw.scales), fw.scale_period, fw.group_size, _ptr(dx), dx_dtype, _ptr(addend),
+                  _ptr(workspace), workspace.numel(), _stream())
+        return dx
     capi.call("caifx_qlinear_backward_input", M, fw.N, fw.K, _ptr(dy), yd, compute_dtype, _ptr(fw.wq),
               fw.w_kind, _ptr(fw.scales), fw.scale_period, fw.group_size, _ptr(dx), dx_dtype,
               _ptr(workspace), workspace.numel(), _stream())
@@ -169,7 +182,7 @@ class GroupedFrozenWeights:
             self.scales_ptrs = torch.tensor([w.scales.data_ptr() for w in weights], dtype=torch.int64, device=dev)
 
 
-def _grouped(name, backward, x, offsets, gw, compute_dtype, out_dtype, out, workspace):
+def _grouped(name, backward, x, offsets, gw, compute_dtype, out_dtype, out, workspace, addend=None):
     _need_cuda(x, offsets)
     in_dim = gw.N if backward else gw.K
     out_dim = gw.K if backward else gw.N
@@ -180,6 +193,12 @@ def _grouped(name, backward, x, offsets, gw, compute_dtype, out_dtype, out, work
     if workspace is None:
         workspace = _workspace(capi.lib().caifx_qlinear_grouped_workspace_bytes(
             E, rows, gw.N, gw.K, xd, compute_dtype, gw.w_kind, int(backward)), x.device)
+    if addend is not None:
+        assert addend.dtype == y.dtype and addend.numel() == y.numel()
+        capi.call(name + "_add", E, _ptr(offsets), rows, gw.N, gw.K, _ptr(x), xd, compute_dtype, _ptr(gw.wq_ptrs),
+                  gw.w_kind, _ptr(gw.scales_ptrs), gw.scale_period, gw.group_size, _ptr(y), out_dtype, _ptr(addend),
+                  _ptr(workspace), workspace.numel(), _stream())
+        return y
     capi.call(name, E, _ptr(offsets), rows, gw.N, gw.K, _ptr(x), xd, compute_dtype, _ptr(gw.wq_ptrs), gw.w_kind,
               _ptr(gw.scales_ptrs), gw.scale_period, gw.group_size, _ptr(y), out_dtype, _ptr(workspace),
               workspace.numel(), _stream())
@@ -190,9 +209,10 @@ def qlinear_grouped_forward(x, offsets, gw, compute_dtype, y_dtype=F32, out=None
     return _grouped("caifx_qlinear_grouped_forward", False, x, offsets, gw, compute_dtype, y_dtype, out, workspace)
 
 
-def qlinear_grouped_backward_input(dy, offsets, gw, compute_dtype, dx_dtype=F32, out=None, workspace=None):
+def qlinear_grouped_backward_input(dy, offsets, gw, compute_dtype, dx_dtype=F32, out=None, workspace=None,
+                                   addend=None):
     return _grouped("caifx_qlinear_grouped_backward_input", True, dy, offsets, gw, compute_dtype, dx_dtype, out,
-                    workspace)
+                    workspace, addend)
 
 
 # ------------------------------------------------------------------ element-wise

@@ -141,7 +141,28 @@ CAIFX_API int caifx_qlinear_backward_input(int64_t M, int64_t N, int64_t K,
                                  void *dx, int dx_dtype,
                                  void *workspace, size_t workspace_bytes, caifx_stream_t stream);
 
-/* Bytes of workspace the two calls above need for this problem (may be 0).
+/* The two calls above followed by the caller's cast to its tensor dtype and an element-wise Add, as
+ * CAIF_DeviceLoRAAdapter composes the frozen base with the low-rank branch
+ * (src/caif_device_lora_adapter.cpp:186-198 forward: base_out.To(StorageT) + lora_out;
+ * :264-276 backward: grad_base.To(StorageT) + d_input_lora):
+ *   y = T(float(T(acc)) + float(addend)),  T = y_dtype, addend [M,N] (forward) / [M,K] (backward) of y_dtype.
+ * The roundings are those of the cast and of the Add, so the bits equal the three-launch sequence.  The
+ * large-M kernels add in their store (the fp32 result and its cast copy never touch memory); other shapes
+ * run the plain call and the Add.  addend must not alias the output. */
+CAIFX_API int caifx_qlinear_forward_add(int64_t M, int64_t N, int64_t K,
+                              const void *x, int x_dtype, int compute_dtype,
+                              const void *wq, int w_kind, const void *scales, int64_t scale_period,
+                              int group_size,
+                              void *y, int y_dtype, const void *addend,
+                              void *workspace, size_t workspace_bytes, caifx_stream_t stream);
+CAIFX_API int caifx_qlinear_backward_input_add(int64_t M, int64_t N, int64_t K,
+                                     const void *dy, int dy_dtype, int compute_dtype,
+                                     const void *wq, int w_kind, const void *scales, int64_t scale_period,
+                                     int group_size,
+                                     void *dx, int dx_dtype, const void *addend,
+                                     void *workspace, size_t workspace_bytes, caifx_stream_t stream);
+
+/* Bytes of workspace the calls above need for this problem (may be 0).
  * backward != 0 asks for caifx_qlinear_backward_input. */
 CAIFX_API size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtype, int compute_dtype,
                                      int w_kind, int backward);
@@ -172,6 +193,19 @@ CAIFX_API int caifx_qlinear_grouped_backward_input(int num_experts, const int32_
                                          int group_size,
                                          void *dx, int dx_dtype,
                                          void *workspace, size_t workspace_bytes, caifx_stream_t stream);
+/* caifx_qlinear_grouped_backward_input with the sum of CAIF_DeviceMoEFrozenExpert::BackwardImpl folded into
+ * its store (src/caif_device_moe_frozen_expert.cpp:291-316: grad_input = gi_up.To(StorageT) +
+ * gi_gate.To(StorageT)): dx[r,:] = T(float(T(dy[r,:] * W_e)) + float(addend[r,:])) for the rows of the segments;
+ * addend [total_rows,K] of dx_dtype, not aliasing dx.  CAIFX_ERR_UNSUPPORTED for shapes the matrix-core kernel
+ * does not take (the caller then uses the plain call and caifx_add). */
+CAIFX_API int caifx_qlinear_grouped_backward_input_add(int num_experts, const int32_t *offsets, int64_t total_rows,
+                                             int64_t N, int64_t K,
+                                             const void *dy, int dy_dtype, int compute_dtype,
+                                             const void *const *wq_ptrs, int w_kind,
+                                             const void *const *scales_ptrs, int64_t scale_period,
+                                             int group_size,
+                                             void *dx, int dx_dtype, const void *addend,
+                                             void *workspace, size_t workspace_bytes, caifx_stream_t stream);
 CAIFX_API size_t caifx_qlinear_grouped_workspace_bytes(int num_experts, int64_t total_rows, int64_t N, int64_t K,
                                              int x_dtype, int compute_dtype, int w_kind, int backward);
 

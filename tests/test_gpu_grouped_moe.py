@@ -210,3 +210,24 @@ def test_fused_swiglu_backward_equals_the_four_op_chain(orc):
         o_gg = orc.silu_backward(gh_, orc.multiply(hh_, uh_, dt), dt)
         assert np.all(np.abs(host(gu) - o_gu) <= ulp * np.maximum(np.abs(o_gu), 1e-3) * 1.01)
         assert np.all(np.abs(host(gg) - o_gg) <= 2 * ulp * np.maximum(np.abs(o_gg), 1e-3) * 1.01)
+
+
+@pytest.mark.parametrize("kind", ["int8pc", "int4"])
+def test_grouped_backward_with_fused_add(orc, kind):
+    # dX = T(T(dY W_e) + addend) per segment equals the plain grouped call followed by Add; rows past the last
+    # segment keep what they held
+    rng = np.random.default_rng(77)
+    E, N, K = 5, 192, 256
+    counts = np.array([130, 0, 77, 257, 3])
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    total = int(offsets[-1])
+    _, gw = _experts(orc, rng, E, N, K, kind, group=64)
+    dy = dev_as(rng.normal(0, 1e-2, (total + 2, N)), 2)
+    addend = dev_as(rng.normal(0, 1e-2, (total + 2, K)), 2)
+    off_d = dev(offsets)
+    plain = T.qlinear_grouped_backward_input(dy, off_d, gw, T.BF16, T.BF16)
+    want = T.add(plain, addend)
+    out = torch.full((total + 2, K), 7.0, dtype=torch.bfloat16, device="cuda")
+    got = T.qlinear_grouped_backward_input(dy, off_d, gw, T.BF16, T.BF16, out=out, addend=addend)
+    assert torch.equal(got[:total], want[:total])
+    assert torch.all(got[total:] == 7.0)
