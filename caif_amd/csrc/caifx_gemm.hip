@@ -59,7 +59,7 @@ struct TileArgs {
   void *d;                   // result [M, C]
   int d_dtype;
   const void *addend;        // optional [M, C] of d_dtype: d = T(float(T(acc)) + float(addend))
-  int vec_store;             // 16-bit result, C % 8 == 0, 16-byte aligned pointers: the store goes through LDS in 16-byte pieces
+  int vec_store;             // C % 8 == 0, 16-byte aligned pointers: the store goes through LDS in 16-byte pieces
   const void *wq;
   const void *scales;
   int group_shift;           // int4: log2(group_size)
@@ -562,51 +562,63 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
   }
 
   // ---- epilogue: acc[i][j][r] = D[row][col], row = 8*(r/4) + 4*(lane/32) + r%4, col = lane%32
-  // 16-bit results: a lane's values sit in 16 different rows, two bytes each, so a direct store moves 64-byte
-  // pieces.  After the last barrier nobody reads the operand tiles any more, so each consumer wave lays its
-  // (BM/2) x 64 sub-tile out in a private piece of LDS (row pitch 144 bytes: conflict free both ways) and
-  // writes it, and reads the optional addend, as 16 bytes per lane and 128 contiguous bytes per row.
+  // A lane's values sit in 16 different rows, one element each, so a direct store moves 64- or 128-byte pieces
+  // with one instruction per element.  After the last barrier nobody reads the operand tiles any more, so each
+  // consumer wave lays its (BM/2) x 64 sub-tile out in a private piece of LDS (row pitch = row + 16 bytes:
+  // conflict free both ways; fp32 in two halves) and writes it, and reads the optional addend, as 16 bytes
+  // per lane and whole 128- or 256-byte row pieces.
   if (g.vec_store) {
-    constexpr int kPitch = 64 * 2 + 16;
-    unsigned char *stage = smem + wave * (kWaveRows * kPitch);
     auto staged = [&](auto tag) {
       typedef decltype(tag) T;
+      constexpr int kPitch = 64 * sizeof(T) + 16;
+      constexpr int kPasses = sizeof(T) == 4 ? 2 : 1;        // fp32: half of the sub-tile's rows at a time
+      constexpr int kRowsPerPass = kWaveRows / kPasses;
+      constexpr int kPer = 16 / sizeof(T);                   // elements per 16-byte piece
+      constexpr int kLanesPerRow = 64 / kPer;
+      unsigned char *stage = smem + wave * (kRowsPerPass * kPitch);
 #pragma unroll
-      for (int i = 0; i < WR; ++i)
+      for (int pass = 0; pass < kPasses; ++pass) {
+        if (pass > 0) asm volatile("" ::: "memory");
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int ii = 0; ii < WR / kPasses; ++ii) {
+          const int i = pass * (WR / kPasses) + ii;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int lrow = i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            *reinterpret_cast<T *>(stage + lrow * kPitch + (j * 32 + (lane & 31)) * 2) = from_f32<T>(acc[i][j][r]);
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int lrow = ii * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+              *reinterpret_cast<T *>(stage + lrow * kPitch + (j * 32 + (lane & 31)) * sizeof(T)) = from_f32<T>(acc[i][j][r]);
+            }
+        }
+        // same wave, LDS executes a wave's accesses in order: only the compiler must not move the reads up
+        asm volatile("" ::: "memory");
+        const int chunk = lane % kLanesPerRow;
+        const int64_t gcol = col0 + wc * 64 + chunk * kPer;
+#pragma unroll
+        for (int it = 0; it < kRowsPerPass * kLanesPerRow / 64; ++it) {
+          const int lrow = it * (64 / kLanesPerRow) + lane / kLanesPerRow;
+          const int64_t grow = row_lo + wm * kWaveRows + pass * kRowsPerPass + lrow;
+          if (grow < row_hi && gcol < C) {
+            u32x4_t v = *reinterpret_cast<const u32x4_t *>(stage + lrow * kPitch + chunk * 16);
+            const int64_t o = grow * C + gcol;
+            if (g.addend) {
+              const u32x4_t av = *reinterpret_cast<const u32x4_t *>(static_cast<const T *>(g.addend) + o);
+              const T *vp = reinterpret_cast<const T *>(&v);
+              const T *ap = reinterpret_cast<const T *>(&av);
+              u32x4_t w;
+              T *wp = reinterpret_cast<T *>(&w);
+#pragma unroll
+              for (int e = 0; e < kPer; ++e) wp[e] = from_f32<T>(to_f32<T>(vp[e]) + to_f32<T>(ap[e]));
+              v = w;
+            }
+            *reinterpret_cast<u32x4_t *>(static_cast<T *>(g.d) + o) = v;
           }
-      // same wave, LDS executes a wave's accesses in order: only the compiler must not move the reads up
-      asm volatile("" ::: "memory");
-      const int chunk = lane & 7;
-      const int64_t gcol = col0 + wc * 64 + chunk * 8;
-#pragma unroll
-      for (int it = 0; it < kWaveRows / 8; ++it) {
-        const int lrow = it * 8 + (lane >> 3);
-        const int64_t grow = row_lo + wm * kWaveRows + lrow;
-        if (grow < row_hi && gcol < C) {
-          u32x4_t v = *reinterpret_cast<const u32x4_t *>(stage + lrow * kPitch + chunk * 16);
-          const int64_t o = grow * C + gcol;
-          if (g.addend) {
-            const u32x4_t av = *reinterpret_cast<const u32x4_t *>(static_cast<const T *>(g.addend) + o);
-            const T *vp = reinterpret_cast<const T *>(&v);
-            const T *ap = reinterpret_cast<const T *>(&av);
-            u32x4_t w;
-            T *wp = reinterpret_cast<T *>(&w);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) wp[e] = from_f32<T>(to_f32(vp[e]) + to_f32(ap[e]));
-            v = w;
-          }
-          *reinterpret_cast<u32x4_t *>(static_cast<T *>(g.d) + o) = v;
         }
       }
     };
     if (g.d_dtype == CAIFX_BF16) staged(bf16_t{});
-    else staged(f16_t{});
+    else if (g.d_dtype == CAIFX_F16) staged(f16_t{});
+    else staged(float{});
     return;
   }
 #pragma unroll
@@ -741,7 +753,7 @@ int run(const GemmArgs &a, bool backward, hipStream_t s)
   t.addend = a.addend;
   {
     const int64_t cols = backward ? a.K : a.N;
-    t.vec_store = a.y_dtype != CAIFX_F32 && cols % 8 == 0 && aligned_to(a.y, 16) && (!a.addend || aligned_to(a.addend, 16));
+    t.vec_store = cols % 8 == 0 && aligned_to(a.y, 16) && (!a.addend || aligned_to(a.addend, 16));
   }
   t.wq = a.w.q;
   t.scales = a.w.scales;
