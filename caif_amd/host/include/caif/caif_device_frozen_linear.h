@@ -18,9 +18,11 @@
 #pragma once
 
 #include <cstdint>
+#include <map>
 #include <memory>
 #include <string>
 #include <type_traits>
+#include <utility>
 #include <vector>
 
 #include "caif_device_frozen_linear_base.h"
@@ -269,6 +271,75 @@ class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
       }
       CAIF_CATCH_BLOCK()
     }
+    // On-disk form of the quantised storage (not in the reference, which exports frozen weights as
+    // fp32 only, src/caif_device_frozen_linear.cpp:760-826): "<prefix>weight" = the codes as they sit
+    // in memory (I8 [OutputDim,InputDim], or I4 of the same shape packed two codes per byte, low
+    // nibble = even flat index) and "<prefix>scales" (F32 [1] or [OutputDim]; F16 [groups]), plus
+    // the three facts a reader needs to interpret them.  The pointers stay owned by the layer.
+    void ExportQuantized(const std::string &prefix,
+                         std::vector<std::pair<std::string,const CAIF_DeviceTensor*>> &tensors,
+                         std::map<std::string,std::string> &metadata)const
+    {
+      try
+      {
+        if(_weight.IsEmpty()==true||_scales.IsEmpty()==true)
+        {
+          THROW_CAIFE("FrozenLinear::ExportQuantized: weight and scales must be loaded (and resident on the device)");
+        }
+        tensors.emplace_back(prefix+"weight",&_weight);
+        tensors.emplace_back(prefix+"scales",&_scales);
+        metadata[prefix+"storage"]=CAIF_DataType(Base_t::StorageDtype()).Name();
+        metadata[prefix+"group_size"]=std::to_string(_group_size);
+        metadata[prefix+"int8_scheme"]=SchemeName(_int8_scheme);
+      }
+      CAIF_CATCH_BLOCK()
+    }
+    // Takes "<prefix>weight" and "<prefix>scales" out of `tensors` (e.g. what
+    // CAIF_SafeTensorsFormat::Load returned) after checking them against this layer: storage type,
+    // shape, group size, int8 scheme, scales length.  Nothing passes through host memory here.
+    void ImportQuantized(const std::string &prefix,std::map<std::string,CAIF_DeviceTensor> &tensors,
+                         const std::map<std::string,std::string> &metadata)
+    {
+      try
+      {
+        auto w=tensors.find(prefix+"weight");
+        auto s=tensors.find(prefix+"scales");
+        if(w==tensors.end()||s==tensors.end())
+        {
+          THROW_CAIFE("FrozenLinear::ImportQuantized: missing tensor "+prefix+(w==tensors.end()?"weight":"scales"));
+        }
+        auto meta=[&](const char *key)
+        {
+          const auto it=metadata.find(prefix+key);
+          if(it==metadata.end())
+          {
+            THROW_CAIFE("FrozenLinear::ImportQuantized: missing metadata "+prefix+key);
+          }
+          return it->second;
+        };
+        if(meta("storage")!=CAIF_DataType(Base_t::StorageDtype()).Name()||w->second.Dtype()!=Base_t::StorageDtype())
+        {
+          THROW_CAIFE("FrozenLinear::ImportQuantized: storage type does not match the layer");
+        }
+        if(IsInt4()==true&&meta("group_size")!=std::to_string(_group_size))
+        {
+          THROW_CAIFE("FrozenLinear::ImportQuantized: group size does not match the layer");
+        }
+        if(IsInt4()==false&&meta("int8_scheme")!=SchemeName(_int8_scheme))
+        {
+          THROW_CAIFE("FrozenLinear::ImportQuantized: int8 scheme does not match the layer");
+        }
+        if(w->second.Shape()!=std::vector<uint32_t>{OutputDim(),InputDim()})
+        {
+          THROW_CAIFE("FrozenLinear::ImportQuantized: weight shape must be [output_dim, input_dim]");
+        }
+        LoadScalesFromTensor(std::move(s->second));
+        LoadFromTensor(std::move(w->second));
+        tensors.erase(prefix+"weight");
+        tensors.erase(prefix+"scales");
+      }
+      CAIF_CATCH_BLOCK()
+    }
     void ClearFP32Cache()override{}
     bool NeedsScales()const override{return true;}
     CAIF_Ops::QuantScheme_e Int8Scheme()const override{return _int8_scheme;}
@@ -343,6 +414,10 @@ class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
 
   private:
     static constexpr bool IsInt4(){return std::is_same<StorageT,caif_int4_packed_t>::value;}
+    static const char *SchemeName(CAIF_Ops::QuantScheme_e s)
+    {
+      return s==CAIF_Ops::QuantScheme_e::PerChannel_e?"per_channel":"per_tensor";
+    }
     const void *ScalesPtr()const{return _scales.IsEmpty()?nullptr:_scales.DeviceDataRaw();}
     void RequireScales()const
     {

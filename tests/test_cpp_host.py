@@ -1,7 +1,7 @@
 """Runs the C++ host-layer test programs (tests/cpp/*.cpp, built by __graft_entry__.build()).
 
 The programs exercise the reference-named classes (CAIF_Ops, CAIF_DeviceFrozenLinear,
-CAIF_DeviceFrozenLinearFactory, CAIF_DeviceMoEFrozenExpert) over the C ABI.  Without a GPU only the
+CAIF_DeviceFrozenLinearFactory, CAIF_DeviceMoEFrozenExpert, CAIF_SafeTensorsFormat) over the C ABI.  Without a GPU only the
 checks that need no device run (`--cpu`); with one, everything."""
 import os
 import subprocess
@@ -9,7 +9,8 @@ import subprocess
 import pytest
 
 BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "bin")
-PROGRAMS = ["test_quantize_ops", "test_device_frozen_linear", "test_device_moe_frozen_expert", "test_moe_routing"]
+PROGRAMS = ["test_quantize_ops", "test_device_frozen_linear", "test_device_moe_frozen_expert", "test_moe_routing",
+            "test_safetensors_quantized"]
 
 
 def _run(name, args):
