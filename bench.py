@@ -297,19 +297,33 @@ def moe_rows(torch, T, dev, gen):
     ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
     state = {}
 
+    hidden, grad_gate, grad_up = bf(rows, H), bf(rows, H), bf(rows, H)
+
     def fwd():
         T.qlinear_grouped_forward(x, offsets, up, T.BF16, T.BF16, out=up_o, workspace=ws)
         T.qlinear_grouped_forward(x, offsets, gate, T.BF16, T.BF16, out=gate_o, workspace=ws)
-        state["hidden"] = T.silu_multiply(gate_o, up_o)
-        T.qlinear_grouped_forward(state["hidden"], offsets, down, T.BF16, T.BF16, out=out, workspace=ws)
+        T.silu_multiply(gate_o, up_o, out=hidden)
+        T.qlinear_grouped_forward(hidden, offsets, down, T.BF16, T.BF16, out=out, workspace=ws)
 
     def bwd():
         T.qlinear_grouped_backward_input(gout, offsets, down, T.BF16, T.BF16, out=gh, workspace=ws)
-        grad_gate, grad_up = T.swiglu_backward(gate_o, up_o, gh)
+        T.swiglu_backward(gate_o, up_o, gh, grad_gate, grad_up)
         T.qlinear_grouped_backward_input(grad_up, offsets, up, T.BF16, T.BF16, out=gi_up, workspace=ws)
         # gi_up + gi_gate folded into the second GEMM's store (same bits as the reference's Add)
         state["dx"] = T.qlinear_grouped_backward_input(grad_gate, offsets, gate, T.BF16, T.BF16, out=gi_gate,
                                                        workspace=ws, addend=gi_up)
+
+    # the same two passes with the gating inside a GEMM's store (same bits, fewer launches and no grad_hidden
+    # buffer; reported beside the separate launches, which are the faster form here)
+    def fwd_gating_in_store():
+        T.qlinear_grouped_forward(x, offsets, gate, T.BF16, T.BF16, out=gate_o, workspace=ws)
+        T.qlinear_grouped_forward_swiglu(x, offsets, up, gate_o, T.BF16, out=(up_o, hidden))
+        T.qlinear_grouped_forward(hidden, offsets, down, T.BF16, T.BF16, out=out, workspace=ws)
+
+    def bwd_gating_in_store():
+        T.qlinear_grouped_backward_input_swiglu(gout, offsets, down, gate_o, up_o, T.BF16, out=(grad_gate, grad_up))
+        T.qlinear_grouped_backward_input(grad_up, offsets, up, T.BF16, T.BF16, out=gi_up, workspace=ws)
+        T.qlinear_grouped_backward_input(grad_gate, offsets, gate, T.BF16, T.BF16, out=gi_gate, workspace=ws, addend=gi_up)
 
     def timed(fn, iters=10):
         fn()
@@ -323,6 +337,7 @@ def moe_rows(torch, T, dev, gen):
         return e0.elapsed_time(e1) / iters
 
     ms_f, ms_b = timed(fwd), timed(bwd)
+    ms_f_fused, ms_b_fused = timed(fwd_gating_in_store), timed(bwd_gating_in_store)
     # token routing around the experts (dispatch map, gather, weighted combine, and their backward passes),
     # on the same routing; HBM-bound row moves: algorithmic bytes = rows read + rows written
     idx2 = ids.reshape(tokens, top_k).to(torch.int32).contiguous()
@@ -359,7 +374,7 @@ def moe_rows(torch, T, dev, gen):
     gemm_flops = 3 * 2.0 * rows * D * H
     return {"experts": E, "tokens": tokens, "top_k": top_k, "packed_rows": rows,
             "rows_per_expert_min_max": [int(counts.min()), int(counts.max())],
-            "fwd_ms": round(ms_f, 4), "bwd_ms": round(ms_b, 4),
+            "fwd_ms": round(ms_f, 4), "bwd_ms": round(ms_b, 4), "gating_in_gemm_store": {"fwd_ms": round(ms_f_fused, 4), "bwd_ms": round(ms_b_fused, 4)},
             "tokens_per_s_fwd_bwd": round(tokens / ((ms_f + ms_b) * 1e-3), 1),
             "routing": routing,
             "tokens_per_s_fwd_bwd_with_routing": round(tokens / ((ms_f + ms_b + routing_ms) * 1e-3), 1),

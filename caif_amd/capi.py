@@ -26,7 +26,8 @@ EXPORTS = [
     "caifx_qlinear_forward", "caifx_qlinear_backward_input", "caifx_qlinear_workspace_bytes",
     "caifx_qlinear_forward_add", "caifx_qlinear_backward_input_add", "caifx_qlinear_grouped_backward_input_add",
     "caifx_qlinear_grouped_forward", "caifx_qlinear_grouped_backward_input",
-    "caifx_qlinear_grouped_workspace_bytes",
+    "caifx_qlinear_grouped_workspace_bytes", "caifx_qlinear_grouped_forward_swiglu",
+    "caifx_qlinear_grouped_backward_input_swiglu",
     "caifx_silu", "caifx_silu_backward", "caifx_multiply", "caifx_add", "caifx_silu_multiply",
     "caifx_swiglu_backward",
     "caifx_moe_dispatch_map_workspace_bytes", "caifx_moe_build_dispatch_map", "caifx_moe_dispatch",
@@ -85,6 +86,8 @@ def lib():
         L.caifx_qlinear_grouped_forward.argtypes = grouped
         L.caifx_qlinear_grouped_backward_input.argtypes = grouped
         L.caifx_qlinear_grouped_backward_input_add.argtypes = grouped[:15] + [_p] + grouped[15:]
+        L.caifx_qlinear_grouped_forward_swiglu.argtypes = grouped[:13] + [_p, _p, _p, _int, _p]
+        L.caifx_qlinear_grouped_backward_input_swiglu.argtypes = grouped[:13] + [_p, _p, _p, _p, _int, _p]
         L.caifx_qlinear_grouped_workspace_bytes.restype = _sz
         L.caifx_qlinear_grouped_workspace_bytes.argtypes = [_int, _i64, _i64, _i64, _int, _int, _int, _int]
         L.caifx_silu.argtypes = [_p, _p, _i64, _int, _p]

@@ -271,4 +271,63 @@ int caifx_qlinear_grouped_backward_input_add(int num_experts, const int32_t *off
                  scales_ptrs, scale_period, group_size, dx, dx_dtype, addend, workspace, workspace_bytes, stream);
 }
 
+// Shared checks of the two gated-expert launches: 16-bit results, every tensor of the result's shape present,
+// aligned to its element type and distinct from the results.
+static int swiglu_grouped(bool backward, int num_experts, const int32_t *offsets, int64_t total_rows, int64_t N, int64_t K,
+                          const void *x, int x_dtype, int compute_dtype, const void *const *wq_ptrs, int w_kind,
+                          const void *const *scales_ptrs, int64_t scale_period, int group_size, const void *gate,
+                          const void *up, void *y, void *y2, int y_dtype, caifx_stream_t stream)
+{
+  int st = validate_common(total_rows, N, K, x, x_dtype, compute_dtype, y, y_dtype);
+  if (st != CAIFX_OK) return st;
+  if (num_experts < 0) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (num_experts == 0 || total_rows == 0) return CAIFX_OK;
+  if (!offsets || !wq_ptrs || !gate || !y2 || (backward && !up)) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (y_dtype != CAIFX_F16 && y_dtype != CAIFX_BF16) return CAIFX_ERR_INVALID_ARGUMENT;
+  if (w_kind == CAIFX_W_INT4_GROUP) {
+    if (group_size <= 0 || !scales_ptrs) return CAIFX_ERR_INVALID_ARGUMENT;
+  } else if (w_kind == CAIFX_W_INT8) {
+    if (scales_ptrs && scale_period <= 0) return CAIFX_ERR_INVALID_ARGUMENT;
+  } else {
+    return CAIFX_ERR_INVALID_ARGUMENT;
+  }
+  if (y == y2 || gate == y || gate == y2 || (backward && (up == y || up == y2)) || x == y || x == y2)
+    return CAIFX_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(gate, 2) || !aligned_to(y2, 2) || (backward && !aligned_to(up, 2))) return CAIFX_ERR_MISALIGNED;
+  GemmArgs a = make_args(total_rows, N, K, x, x_dtype, compute_dtype, nullptr, w_kind, nullptr, scale_period,
+                         group_size, y, y_dtype, nullptr, 0);
+  a.w.scale_period = (w_kind == CAIFX_W_INT8 && scales_ptrs) ? scale_period : 1;
+  a.offsets = offsets;
+  a.wq_ptrs = wq_ptrs;
+  a.scales_ptrs = scales_ptrs;
+  a.num_experts = num_experts;
+  a.epilogue = backward ? 2 : 1;
+  a.e1 = gate;
+  a.e2 = up;
+  a.y2 = y2;
+  hipStream_t s = as_stream(stream);
+  return backward ? mfma_backward(a, s) : mfma_forward(a, s);
+}
+
+int caifx_qlinear_grouped_forward_swiglu(int num_experts, const int32_t *offsets, int64_t total_rows, int64_t N, int64_t K,
+                                         const void *x, int x_dtype, int compute_dtype, const void *const *wq_ptrs,
+                                         int w_kind, const void *const *scales_ptrs, int64_t scale_period,
+                                         int group_size, const void *gate, void *up, void *hidden, int out_dtype,
+                                         caifx_stream_t stream)
+{
+  return swiglu_grouped(false, num_experts, offsets, total_rows, N, K, x, x_dtype, compute_dtype, wq_ptrs, w_kind,
+                        scales_ptrs, scale_period, group_size, gate, nullptr, up, hidden, out_dtype, stream);
+}
+
+int caifx_qlinear_grouped_backward_input_swiglu(int num_experts, const int32_t *offsets, int64_t total_rows, int64_t N,
+                                                int64_t K, const void *dy, int dy_dtype, int compute_dtype,
+                                                const void *const *wq_ptrs, int w_kind,
+                                                const void *const *scales_ptrs, int64_t scale_period, int group_size,
+                                                const void *gate, const void *up, void *grad_gate, void *grad_up,
+                                                int out_dtype, caifx_stream_t stream)
+{
+  return swiglu_grouped(true, num_experts, offsets, total_rows, N, K, dy, dy_dtype, compute_dtype, wq_ptrs, w_kind,
+                        scales_ptrs, scale_period, group_size, gate, up, grad_gate, grad_up, out_dtype, stream);
+}
+
 }  // extern "C"

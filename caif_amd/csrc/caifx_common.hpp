@@ -46,6 +46,30 @@ template <typename T> __device__ __forceinline__ float to_f32(T v) { return stat
 template <typename T> __device__ __forceinline__ float round_through(float v) { return to_f32<T>(from_f32<T>(v)); }
 template <> __device__ __forceinline__ float round_through<float>(float v) { return v; }
 
+// SiLU and its derivative (src/caif_cuda_kernels_activations.cu:513-514,558-561), shared by the element-wise
+// kernels and the GEMM epilogues.  The one place where the compiler could choose between a fused and an
+// unfused multiply-add is written out, so every user returns the same bits.
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float silu_bwd_f32(float x, float g)
+{
+  const float s = 1.0f / (1.0f + expf(-x));
+  return g * s * __builtin_fmaf(x, 1.0f - s, 1.0f);
+}
+// One element of the gated expert's backward between its down and up/gate projections
+// (src/caif_device_moe_frozen_expert.cpp:252-290): h = grad of hidden, gate/up = the forward's projections,
+// all already rounded to T; grad_up = T(h * T(silu(gate))), grad_gate = T(silu'(gate) * T(h * up)).
+template <typename T> __device__ __forceinline__ void swiglu_bwd_one(T gate, T up, T h, T &grad_gate, T &grad_up)
+{
+  const float g = to_f32<T>(gate), u = to_f32<T>(up), hh = to_f32<T>(h);
+  grad_up = from_f32<T>(hh * round_through<T>(silu_f32(g)));
+  grad_gate = from_f32<T>(silu_bwd_f32(g, round_through<T>(hh * u)));
+}
+// hidden = T(T(silu(gate)) * up) (:119-153)
+template <typename T> __device__ __forceinline__ T swiglu_fwd_one(T gate, T up)
+{
+  return from_f32<T>(round_through<T>(silu_f32(to_f32<T>(gate))) * to_f32<T>(up));
+}
+
 // Byte k of a dword as fp32 (v_cvt_f32_ubyteK: one VALU op, no shift/mask).
 __device__ __forceinline__ float ubyte0_f32(uint32_t v) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(v)); return r; }
 __device__ __forceinline__ float ubyte1_f32(uint32_t v) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(v)); return r; }

@@ -12,14 +12,10 @@ constexpr int kBlock = 256;
 constexpr int kVec = 8;
 
 struct SiluOp {
-  __device__ float operator()(float x, float) const { return x / (1.0f + expf(-x)); }
+  __device__ float operator()(float x, float) const { return silu_f32(x); }
 };
 struct SiluBwdOp {   // a = forward input x, b = upstream gradient
-  __device__ float operator()(float x, float g) const
-  {
-    const float s = 1.0f / (1.0f + expf(-x));
-    return g * s * (1.0f + x * (1.0f - s));
-  }
+  __device__ float operator()(float x, float g) const { return silu_bwd_f32(x, g); }
 };
 struct MulOp {
   __device__ float operator()(float a, float b) const { return a * b; }
@@ -28,7 +24,7 @@ struct AddOp {
   __device__ float operator()(float a, float b) const { return a + b; }
 };
 template <typename T> struct SiluMulOp {   // a = gate, b = up; silu(gate) is rounded to T first
-  __device__ float operator()(float g, float u) const { return round_through<T>(g / (1.0f + expf(-g))) * u; }
+  __device__ float operator()(float g, float u) const { return round_through<T>(silu_f32(g)) * u; }
 };
 
 template <typename T, typename Op, bool kBinary>
@@ -76,13 +72,7 @@ __global__ void swiglu_bwd_kernel(const T *__restrict__ gate, const T *__restric
                                   T *__restrict__ grad_gate, T *__restrict__ grad_up, int64_t n, int64_t n_body)
 {
   const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  auto one = [&](T g16, T u16, T h16, T &gg, T &gu) {
-    const float g = to_f32<T>(g16), u = to_f32<T>(u16), h = to_f32<T>(h16);
-    const float act = round_through<T>(SiluOp{}(g, 0.0f));
-    gu = from_f32<T>(MulOp{}(h, act));
-    const float tt = round_through<T>(MulOp{}(h, u));
-    gg = from_f32<T>(SiluBwdOp{}(g, tt));
-  };
+  auto one = [&](T g16, T u16, T h16, T &gg, T &gu) { swiglu_bwd_one<T>(g16, u16, h16, gg, gu); };
   const int64_t i = t * kVec;
   if (i < n_body) {
     T vg[kVec], vu[kVec], vh[kVec], og[kVec], ou[kVec];

@@ -52,6 +52,11 @@ template <> struct Mfma32<f16_t> {
 };
 
 enum { SM_SCALAR = 0, SM_VEC4 = 1, SM_ANY = 2 };   // how int8 scales are fetched
+// What the store does besides rounding the accumulator v to the result type T:
+//   EPI_SWIGLU_FWD  the launch is the up projection: d = v, d2 = T(T(silu(e1)) * v)             (e1 = gate)
+//   EPI_SWIGLU_BWD  the launch is the input gradient of the down projection, v = grad of hidden:
+//                   d = T(silu'(e1) * T(v * e2)), d2 = T(v * T(silu(e1)))                       (e1 = gate, e2 = up)
+enum { EPI_NONE = 0, EPI_SWIGLU_FWD = 1, EPI_SWIGLU_BWD = 2 };
 
 struct TileArgs {
   int64_t M, N, K;           // N = OutputDim, K = InputDim of the weight
@@ -60,6 +65,10 @@ struct TileArgs {
   int d_dtype;
   const void *addend;        // optional [M, C] of d_dtype: d = T(float(T(acc)) + float(addend))
   int vec_store;             // C % 8 == 0, 16-byte aligned pointers: the store goes through LDS in 16-byte pieces
+  // gated-expert epilogues (16-bit results through the staged store only), see EPI_*
+  int epilogue;
+  const void *e1, *e2;       // [M, C] of d_dtype: gate (forward); gate, up (backward)
+  void *d2;                  // second result [M, C]
   const void *wq;
   const void *scales;
   int group_shift;           // int4: log2(group_size)
@@ -601,6 +610,28 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
           if (grow < row_hi && gcol < C) {
             u32x4_t v = *reinterpret_cast<const u32x4_t *>(stage + lrow * kPitch + chunk * 16);
             const int64_t o = grow * C + gcol;
+            if constexpr (sizeof(T) == 2 && kGrouped) {        // only the grouped launches carry these
+              if (g.epilogue != EPI_NONE) {
+                const u32x4_t gv = *reinterpret_cast<const u32x4_t *>(static_cast<const T *>(g.e1) + o);
+                const T *vp = reinterpret_cast<const T *>(&v);
+                const T *gp = reinterpret_cast<const T *>(&gv);
+                u32x4_t w1 = v, w2;
+                T *p1 = reinterpret_cast<T *>(&w1);
+                T *p2 = reinterpret_cast<T *>(&w2);
+                if (g.epilogue == EPI_SWIGLU_FWD) {
+#pragma unroll
+                  for (int e = 0; e < kPer; ++e) p2[e] = swiglu_fwd_one<T>(gp[e], vp[e]);
+                } else {
+                  const u32x4_t uv = *reinterpret_cast<const u32x4_t *>(static_cast<const T *>(g.e2) + o);
+                  const T *up = reinterpret_cast<const T *>(&uv);
+#pragma unroll
+                  for (int e = 0; e < kPer; ++e) swiglu_bwd_one<T>(gp[e], up[e], vp[e], p1[e], p2[e]);
+                }
+                *reinterpret_cast<u32x4_t *>(static_cast<T *>(g.d) + o) = w1;
+                *reinterpret_cast<u32x4_t *>(static_cast<T *>(g.d2) + o) = w2;
+                continue;
+              }
+            }
             if (g.addend) {
               const u32x4_t av = *reinterpret_cast<const u32x4_t *>(static_cast<const T *>(g.addend) + o);
               const T *vp = reinterpret_cast<const T *>(&v);
@@ -754,6 +785,16 @@ int run(const GemmArgs &a, bool backward, hipStream_t s)
   {
     const int64_t cols = backward ? a.K : a.N;
     t.vec_store = cols % 8 == 0 && aligned_to(a.y, 16) && (!a.addend || aligned_to(a.addend, 16));
+  }
+  if (a.epilogue != EPI_NONE) {
+    // only the staged 16-byte store carries these; the caller falls back to separate launches otherwise
+    if (!grouped || !t.vec_store || a.y_dtype == CAIFX_F32 || a.addend || !aligned_to(a.e1, 16) || !aligned_to(a.y2, 16) ||
+        (a.epilogue == EPI_SWIGLU_BWD && !aligned_to(a.e2, 16)))
+      return CAIFX_ERR_UNSUPPORTED;
+    t.epilogue = a.epilogue;
+    t.e1 = a.e1;
+    t.e2 = a.e2;
+    t.d2 = a.y2;
   }
   t.wq = a.w.q;
   t.scales = a.w.scales;

@@ -31,6 +31,11 @@ struct GemmArgs {
   size_t workspace_bytes;
   // optional: y = T(float(T(acc)) + float(addend)), addend [M, columns of y] of y_dtype (may alias y)
   const void *addend;
+  // optional gated-expert epilogue of the matrix-core kernel (0 = none, 1 = forward, 2 = backward; see
+  // EPI_* in caifx_gemm.hip): e1 = gate, e2 = up (backward only), y2 = second result, all [M, columns of y]
+  int epilogue;
+  const void *e1, *e2;
+  void *y2;
 };
 
 int generic_forward(const GemmArgs &a, hipStream_t s);

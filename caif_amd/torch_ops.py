@@ -215,10 +215,36 @@ def qlinear_grouped_backward_input(dy, offsets, gw, compute_dtype, dx_dtype=F32,
                     workspace, addend)
 
 
+def qlinear_grouped_forward_swiglu(x, offsets, gw_up, gate, compute_dtype, out=None):
+    """Up projection with the gating in its store: returns (up, hidden), both of gate's dtype and shape."""
+    _need_cuda(x, offsets, gate)
+    rows = x.numel() // gw_up.K
+    up, hidden = out if out is not None else (torch.zeros_like(gate), torch.zeros_like(gate))
+    capi.call("caifx_qlinear_grouped_forward_swiglu", len(gw_up.weights), _ptr(offsets), rows, gw_up.N, gw_up.K, _ptr(x),
+              CODE_OF[x.dtype], compute_dtype, _ptr(gw_up.wq_ptrs), gw_up.w_kind, _ptr(gw_up.scales_ptrs),
+              gw_up.scale_period, gw_up.group_size, _ptr(gate), _ptr(up), _ptr(hidden), CODE_OF[gate.dtype], _stream())
+    return up, hidden
+
+
+def qlinear_grouped_backward_input_swiglu(dy, offsets, gw_down, gate, up, compute_dtype, out=None):
+    """Input gradient of the down projection with the gating's backward in its store: returns (grad_gate, grad_up)."""
+    _need_cuda(dy, offsets, gate, up)
+    rows = dy.numel() // gw_down.N
+    grad_gate, grad_up = out if out is not None else (torch.zeros_like(gate), torch.zeros_like(gate))
+    capi.call("caifx_qlinear_grouped_backward_input_swiglu", len(gw_down.weights), _ptr(offsets), rows, gw_down.N, gw_down.K,
+              _ptr(dy), CODE_OF[dy.dtype], compute_dtype, _ptr(gw_down.wq_ptrs), gw_down.w_kind, _ptr(gw_down.scales_ptrs),
+              gw_down.scale_period, gw_down.group_size, _ptr(gate), _ptr(up), _ptr(grad_gate), _ptr(grad_up),
+              CODE_OF[gate.dtype], _stream())
+    return grad_gate, grad_up
+
+
 # ------------------------------------------------------------------ element-wise
-def _ew(name, n_in, a, b=None):
-    _need_cuda(a, b)
-    out = torch.empty_like(a)
+def _ew(name, n_in, a, b=None, out=None):
+    _need_cuda(a, b, out)
+    if out is None:
+        out = torch.empty_like(a)
+    elif out.dtype != a.dtype or out.numel() != a.numel() or not out.is_contiguous():
+        raise ValueError("out must be a contiguous tensor of the input's dtype and size")
     dt = CODE_OF[a.dtype]
     if n_in == 1:
         capi.call(name, _ptr(a), _ptr(out), a.numel(), dt, _stream())
@@ -243,8 +269,8 @@ def add(a, b):
     return _ew("caifx_add", 2, a, b)
 
 
-def silu_multiply(gate, up):
-    return _ew("caifx_silu_multiply", 2, gate, up)
+def silu_multiply(gate, up, out=None):
+    return _ew("caifx_silu_multiply", 2, gate, up, out)
 
 
 def swiglu_backward(gate, up, grad_hidden, out_gate=None, out_up=None):

@@ -206,6 +206,35 @@ CAIFX_API int caifx_qlinear_grouped_backward_input_add(int num_experts, const in
                                              int group_size,
                                              void *dx, int dx_dtype, const void *addend,
                                              void *workspace, size_t workspace_bytes, caifx_stream_t stream);
+/* The up projection of CAIF_DeviceMoEFrozenExpert::ForwardImpl with the expert's gating folded into its store
+ * (src/caif_device_moe_frozen_expert.cpp:119-153: up_out.To(StorageT); SiLU(gate); Multiply): for the rows of
+ * the segments up[r,:] = T(x[r,:] * W_e^T) and hidden[r,:] = T(T(silu(gate[r,:])) * up[r,:]), with the cast
+ * points of the three separate launches (the result equals caifx_qlinear_grouped_forward followed by
+ * caifx_silu_mul bit for bit).  gate, up, hidden: [total_rows,N] of out_dtype (CAIFX_F16 or CAIFX_BF16),
+ * pairwise distinct.  CAIFX_ERR_UNSUPPORTED for shapes the matrix-core kernel does not take or results that
+ * are not 16-byte aligned with N % 8 == 0 (the caller then uses the separate calls).  This form and the one
+ * below save a launch and, in the backward, the grad-of-hidden buffer; at 64 experts x 24576 rows (2048 <-> 1408)
+ * they measure 4 % / 10 % slower than the separate launches, whose element-wise pass runs at full occupancy. */
+CAIFX_API int caifx_qlinear_grouped_forward_swiglu(int num_experts, const int32_t *offsets, int64_t total_rows,
+                                         int64_t N, int64_t K,
+                                         const void *x, int x_dtype, int compute_dtype,
+                                         const void *const *wq_ptrs, int w_kind,
+                                         const void *const *scales_ptrs, int64_t scale_period, int group_size,
+                                         const void *gate, void *up, void *hidden, int out_dtype,
+                                         caifx_stream_t stream);
+/* The input gradient of the down projection in CAIF_DeviceMoEFrozenExpert::BackwardImpl with the gating's
+ * backward folded into its store (src/caif_device_moe_frozen_expert.cpp:252-290): with h = T(dy[r,:] * W_e)
+ * (never written), grad_up[r,:] = T(h * T(silu(gate[r,:]))) and grad_gate[r,:] = T(silu'(gate[r,:]) * T(h * up[r,:]))
+ * (equal to caifx_qlinear_grouped_backward_input followed by caifx_swiglu_backward bit for bit).  gate, up,
+ * grad_gate, grad_up: [total_rows,K] of out_dtype (16-bit), pairwise distinct.  CAIFX_ERR_UNSUPPORTED as above. */
+CAIFX_API int caifx_qlinear_grouped_backward_input_swiglu(int num_experts, const int32_t *offsets, int64_t total_rows,
+                                                int64_t N, int64_t K,
+                                                const void *dy, int dy_dtype, int compute_dtype,
+                                                const void *const *wq_ptrs, int w_kind,
+                                                const void *const *scales_ptrs, int64_t scale_period,
+                                                int group_size,
+                                                const void *gate, const void *up, void *grad_gate, void *grad_up,
+                                                int out_dtype, caifx_stream_t stream);
 CAIFX_API size_t caifx_qlinear_grouped_workspace_bytes(int num_experts, int64_t total_rows, int64_t N, int64_t K,
                                              int x_dtype, int compute_dtype, int w_kind, int backward);
 

@@ -345,7 +345,9 @@ ORC_API void orc_silu(const float *in, float *out, int64_t n, int dtype)
 
 /* SiLU backward (src/caif_cuda_kernels_activations.cu:558-561):
  * s = 1/(1+exp(-x)); r = g*s*(1+x*(1-s)), left-to-right fp32, one rounding to
- * the tensor dtype. */
+ * the tensor dtype.  The reference's build leaves nvcc's multiply-add contraction
+ * on (CMakeLists.txt:350-351 sets no --fmad), so 1+x*(1-s) is one fused
+ * multiply-add there; fmaf states that here, whatever -ffp-contract says. */
 ORC_API void orc_silu_backward(const float *x_in, const float *grad_out, float *grad_in, int64_t n, int dtype)
 {
 #pragma omp parallel for schedule(static)
@@ -353,7 +355,7 @@ ORC_API void orc_silu_backward(const float *x_in, const float *grad_out, float *
     float gv = grad_out[i];
     float x = x_in[i];
     float s = 1.0f / (1.0f + expf(-x));
-    grad_in[i] = orc_round_scalar(gv * s * (1.0f + x * (1.0f - s)), dtype);
+    grad_in[i] = orc_round_scalar(gv * s * fmaf(x, 1.0f - s, 1.0f), dtype);
   }
 }
 

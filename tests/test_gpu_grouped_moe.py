@@ -179,11 +179,14 @@ def test_elementwise_ops_match_oracle(orc):
         ah, bh = host(ad), host(bd)
         # expf differs by a few ulp between libm and the device: allow one ulp of the tensor dtype
         ulp = {0: 2e-6, 1: 2 ** -10, 2: 2 ** -7}[dt]
-        for got, want in ((T.silu(ad), orc.silu(ah, dt)),
-                          (T.silu_backward(ad, bd), orc.silu_backward(ah, bh, dt)),
-                          (T.silu_multiply(ad, bd), orc.multiply(orc.silu(ah, dt), bh, dt))):
+        # silu'(x) = s * (1 + x * (1 - s)) cancels near x = -1.278: there the few-ulp difference in s is an
+        # absolute error of that size in the bracket, so its bound is relative to |grad_out|, not to the result
+        for got, want, scale in ((T.silu(ad), orc.silu(ah, dt), None),
+                                 (T.silu_backward(ad, bd), orc.silu_backward(ah, bh, dt), np.abs(bh)),
+                                 (T.silu_multiply(ad, bd), orc.multiply(orc.silu(ah, dt), bh, dt), None)):
             g, w = host(got), want
-            assert np.all(np.abs(g - w) <= ulp * np.maximum(np.abs(w), 1e-3) * 1.01)
+            ref = np.maximum(np.abs(w), 1e-3) if scale is None else np.maximum(np.abs(w), scale)
+            assert np.all(np.abs(g - w) <= ulp * ref * 1.01)
         assert np.array_equal(host(T.multiply(ad, bd)), orc.multiply(ah, bh, dt))   # exact
         assert np.array_equal(host(T.add(ad, bd)), orc.add(ah, bh, dt))             # exact
 
@@ -231,3 +234,50 @@ def test_grouped_backward_with_fused_add(orc, kind):
     got = T.qlinear_grouped_backward_input(dy, off_d, gw, T.BF16, T.BF16, out=out, addend=addend)
     assert torch.equal(got[:total], want[:total])
     assert torch.all(got[total:] == 7.0)
+
+
+@pytest.mark.parametrize("kind", ["int8pc", "int4"])
+@pytest.mark.parametrize("dt", [2, 1])
+def test_grouped_gemm_with_gating_in_its_store(orc, kind, dt):
+    # The up projection that also writes hidden = T(T(silu(gate)) * up), and the down projection's input
+    # gradient that writes grad_gate / grad_up instead of grad_hidden: same bits as the separate launches
+    # (src/caif_device_moe_frozen_expert.cpp:119-153,252-290 fix the cast points); rows past the last segment
+    # keep what they held
+    rng = np.random.default_rng(91 + dt)
+    E, D, H = 6, 256, 192
+    counts = np.array([130, 0, 1, 257, 64, 5])
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    total = int(offsets[-1])
+    _, up_g = _experts(orc, rng, E, H, D, kind, group=64)
+    _, down_g = _experts(orc, rng, E, D, H, kind, group=64)
+    tdt = {1: torch.float16, 2: torch.bfloat16}[dt]
+    x = dev_as(rng.normal(0, 1, (total + 2, D)), dt)
+    gate = dev_as(rng.normal(0, 2, (total + 2, H)), dt)
+    off_d = dev(offsets)
+    want_up = T.qlinear_grouped_forward(x, off_d, up_g, dt, dt)
+    want_hidden = T.silu_multiply(gate, want_up)
+    up, hidden = T.qlinear_grouped_forward_swiglu(x, off_d, up_g, gate, dt)
+    assert torch.equal(up[:total], want_up[:total])
+    assert torch.equal(hidden[:total], want_hidden[:total])
+    assert not up[total:].any() and not hidden[total:].any()
+
+    dy = dev_as(rng.normal(0, 1e-2, (total + 2, D)), dt)
+    gh = T.qlinear_grouped_backward_input(dy, off_d, down_g, dt, dt)
+    want_gg, want_gu = T.swiglu_backward(gate, up, gh)
+    out = (torch.full((total + 2, H), 7.0, dtype=tdt, device="cuda"), torch.full((total + 2, H), 5.0, dtype=tdt, device="cuda"))
+    gg, gu = T.qlinear_grouped_backward_input_swiglu(dy, off_d, down_g, gate, up, dt, out=out)
+    assert torch.equal(gg[:total], want_gg[:total])
+    assert torch.equal(gu[:total], want_gu[:total])
+    assert torch.all(gg[total:] == 7.0) and torch.all(gu[total:] == 5.0)
+
+
+def test_grouped_gemm_gating_refuses_what_the_staged_store_cannot_take(orc):
+    from caif_amd import capi
+    rng = np.random.default_rng(5)
+    E, D, H = 2, 256, 100                                            # H % 8 != 0: no 16-byte store
+    offsets = np.array([0, 40, 90], np.int32)
+    _, up_g = _experts(orc, rng, E, H, D, "int8pc")
+    x = dev_as(rng.normal(0, 1, (90, D)), 2)
+    gate = dev_as(rng.normal(0, 1, (90, H)), 2)
+    with pytest.raises(capi.CaifxError):
+        T.qlinear_grouped_forward_swiglu(x, dev(offsets), up_g, gate, 2)
