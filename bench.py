@@ -325,16 +325,22 @@ def moe_rows(torch, T, dev, gen):
         T.qlinear_grouped_backward_input(grad_up, offsets, up, T.BF16, T.BF16, out=gi_up, workspace=ws)
         T.qlinear_grouped_backward_input(grad_gate, offsets, gate, T.BF16, T.BF16, out=gi_gate, workspace=ws, addend=gi_up)
 
-    def timed(fn, iters=10):
-        fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
+    def timed(fn, iters=10, reps=3):
+        """Milliseconds per call: median of reps event-timed runs of iters eager calls, after iters untimed
+        ones (the first few calls after the one-off quantisation above run at a lower clock)."""
         for _ in range(iters):
             fn()
-        e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / iters
+        times = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1) / iters)
+        return sorted(times)[len(times) // 2]
 
     ms_f, ms_b = timed(fwd), timed(bwd)
     ms_f_fused, ms_b_fused = timed(fwd_gating_in_store), timed(bwd_gating_in_store)

@@ -214,7 +214,8 @@ CAIFX_API int caifx_qlinear_grouped_backward_input_add(int num_experts, const in
  * pairwise distinct.  CAIFX_ERR_UNSUPPORTED for shapes the matrix-core kernel does not take or results that
  * are not 16-byte aligned with N % 8 == 0 (the caller then uses the separate calls).  This form and the one
  * below save a launch and, in the backward, the grad-of-hidden buffer; at 64 experts x 24576 rows (2048 <-> 1408)
- * they measure 4 % / 10 % slower than the separate launches, whose element-wise pass runs at full occupancy. */
+ * an expert pass built on them measures 1-2 % slower than one built on the separate launches, whose
+ * element-wise pass runs at full occupancy. */
 CAIFX_API int caifx_qlinear_grouped_forward_swiglu(int num_experts, const int32_t *offsets, int64_t total_rows,
                                          int64_t N, int64_t K,
                                          const void *x, int x_dtype, int compute_dtype,
