@@ -96,6 +96,17 @@ template <typename CT> __device__ __forceinline__ uint32_t pack2(float lo, float
   return __builtin_bit_cast(uint32_t, p);
 }
 
+// Rows [lo, hi) of expert e, forced into 0 <= lo <= hi <= M: offsets that are not non-decreasing or that
+// run past the buffer (a caller's mistake) then lose rows instead of sending loads and stores out of bounds.
+__device__ __forceinline__ void segment_rows(const int32_t *offsets, int e, int64_t M, int &lo, int &hi)
+{
+  const int m = static_cast<int>(M);          // M <= 2^30 is checked on the host
+  lo = offsets[e];
+  hi = offsets[e + 1];
+  lo = lo < 0 ? 0 : (lo > m ? m : lo);
+  hi = hi < lo ? lo : (hi > m ? m : hi);
+}
+
 __device__ __forceinline__ float int8_scale_at(const float *scales, int mode, int64_t period, int64_t flat)
 {
   if (mode == SM_SCALAR) return scales ? scales[0] : 1.0f;
@@ -150,7 +161,11 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
     for (int base = 0; base < g.num_experts; base += 64) {
       const int my = base + lane;
       int tiles = 0;
-      if (my < g.num_experts) tiles = (g.offsets[my + 1] - g.offsets[my] + BM - 1) / BM;
+      if (my < g.num_experts) {
+        int slo, shi;
+        segment_rows(g.offsets, my, g.M, slo, shi);
+        tiles = (shi - slo + BM - 1) / BM;
+      }
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) tiles += __shfl_xor(tiles, o, 64);
       total_rt += tiles;
@@ -168,10 +183,7 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
     for (int base = 0; base < g.num_experts && !found; base += 64) {
       const int my = base + lane;
       int my_lo = 0, my_hi = 0;
-      if (my < g.num_experts) {
-        my_lo = g.offsets[my];
-        my_hi = g.offsets[my + 1];
-      }
+      if (my < g.num_experts) segment_rows(g.offsets, my, g.M, my_lo, my_hi);
       const int tiles = (my_hi - my_lo + BM - 1) / BM;
       int incl = tiles;
 #pragma unroll

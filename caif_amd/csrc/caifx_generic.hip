@@ -59,6 +59,9 @@ __global__ void generic_forward_kernel(GemmArgs a)
     const int e = blockIdx.z;
     row_lo = a.offsets[e];
     row_hi = a.offsets[e + 1];
+    // offsets that are not non-decreasing or run past the buffer lose rows instead of leaving it
+    row_lo = row_lo < 0 ? 0 : (row_lo > a.M ? a.M : row_lo);
+    row_hi = row_hi < row_lo ? row_lo : (row_hi > a.M ? a.M : row_hi);
     wq = a.wq_ptrs[e];
     scales = a.scales_ptrs ? a.scales_ptrs[e] : nullptr;
   }
@@ -94,6 +97,9 @@ __global__ void generic_backward_kernel(GemmArgs a)
     const int e = blockIdx.z;
     row_lo = a.offsets[e];
     row_hi = a.offsets[e + 1];
+    // offsets that are not non-decreasing or run past the buffer lose rows instead of leaving it
+    row_lo = row_lo < 0 ? 0 : (row_lo > a.M ? a.M : row_lo);
+    row_hi = row_hi < row_lo ? row_lo : (row_hi > a.M ? a.M : row_hi);
     wq = a.wq_ptrs[e];
     scales = a.scales_ptrs ? a.scales_ptrs[e] : nullptr;
   }

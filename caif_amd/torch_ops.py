@@ -182,6 +182,18 @@ class GroupedFrozenWeights:
             self.scales_ptrs = torch.tensor([w.scales.data_ptr() for w in weights], dtype=torch.int64, device=dev)
 
 
+def _check_grouped(x, in_dim, rows, offsets, E, results, out_dim, out_dtype):
+    """The C ABI sees raw pointers: sizes and dtypes are checked here, before anything is launched."""
+    if x.numel() != rows * in_dim:
+        raise ValueError(f"input has {x.numel()} elements, not a multiple of the reduction length {in_dim}")
+    if offsets.dtype != torch.int32 or offsets.numel() != E + 1:
+        raise ValueError(f"offsets must be int32 [{E + 1}]")
+    for t in results:
+        _need_cuda(t)
+        if t.dtype != out_dtype or t.numel() != rows * out_dim:
+            raise ValueError(f"result / gating tensors must be {out_dtype} with {rows} x {out_dim} elements")
+
+
 def _grouped(name, backward, x, offsets, gw, compute_dtype, out_dtype, out, workspace, addend=None):
     _need_cuda(x, offsets)
     in_dim = gw.N if backward else gw.K
@@ -190,6 +202,7 @@ def _grouped(name, backward, x, offsets, gw, compute_dtype, out_dtype, out, work
     y = out if out is not None else torch.zeros((rows, out_dim), dtype=TORCH_DTYPE[out_dtype], device=x.device)
     xd = CODE_OF[x.dtype]
     E = len(gw.weights)
+    _check_grouped(x, in_dim, rows, offsets, E, (y,), out_dim, TORCH_DTYPE[out_dtype])
     if workspace is None:
         workspace = _workspace(capi.lib().caifx_qlinear_grouped_workspace_bytes(
             E, rows, gw.N, gw.K, xd, compute_dtype, gw.w_kind, int(backward)), x.device)
@@ -220,6 +233,7 @@ def qlinear_grouped_forward_swiglu(x, offsets, gw_up, gate, compute_dtype, out=N
     _need_cuda(x, offsets, gate)
     rows = x.numel() // gw_up.K
     up, hidden = out if out is not None else (torch.zeros_like(gate), torch.zeros_like(gate))
+    _check_grouped(x, gw_up.K, rows, offsets, len(gw_up.weights), (gate, up, hidden), gw_up.N, gate.dtype)
     capi.call("caifx_qlinear_grouped_forward_swiglu", len(gw_up.weights), _ptr(offsets), rows, gw_up.N, gw_up.K, _ptr(x),
               CODE_OF[x.dtype], compute_dtype, _ptr(gw_up.wq_ptrs), gw_up.w_kind, _ptr(gw_up.scales_ptrs),
               gw_up.scale_period, gw_up.group_size, _ptr(gate), _ptr(up), _ptr(hidden), CODE_OF[gate.dtype], _stream())
@@ -231,6 +245,7 @@ def qlinear_grouped_backward_input_swiglu(dy, offsets, gw_down, gate, up, comput
     _need_cuda(dy, offsets, gate, up)
     rows = dy.numel() // gw_down.N
     grad_gate, grad_up = out if out is not None else (torch.zeros_like(gate), torch.zeros_like(gate))
+    _check_grouped(dy, gw_down.N, rows, offsets, len(gw_down.weights), (gate, up, grad_gate, grad_up), gw_down.K, gate.dtype)
     capi.call("caifx_qlinear_grouped_backward_input_swiglu", len(gw_down.weights), _ptr(offsets), rows, gw_down.N, gw_down.K,
               _ptr(dy), CODE_OF[dy.dtype], compute_dtype, _ptr(gw_down.wq_ptrs), gw_down.w_kind, _ptr(gw_down.scales_ptrs),
               gw_down.scale_period, gw_down.group_size, _ptr(gate), _ptr(up), _ptr(grad_gate), _ptr(grad_up),

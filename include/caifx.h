@@ -175,7 +175,9 @@ CAIFX_API size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, 
  *   forward : y[r,:] = x[r,:] * W_e^T      x [total_rows,K], y [total_rows,N]
  *   backward: dx[r,:] = dy[r,:] * W_e      dy [total_rows,N], dx [total_rows,K]
  * offsets: device int32[E+1], non-decreasing, offsets[E] <= total_rows (rows
- * past offsets[E] are left untouched).  wq_ptrs / scales_ptrs: device arrays of
+ * past offsets[E] are left untouched; offsets that break this are cut to
+ * 0 <= lo <= hi <= total_rows per expert on the device: rows are lost, nothing
+ * outside the buffers is touched).  wq_ptrs / scales_ptrs: device arrays of
  * E device pointers (one frozen linear per expert, each its own allocation as
  * in the reference); every expert shares N, K, kind, scale_period, group_size. */
 CAIFX_API int caifx_qlinear_grouped_forward(int num_experts, const int32_t *offsets, int64_t total_rows,

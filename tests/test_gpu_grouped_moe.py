@@ -281,3 +281,21 @@ def test_grouped_gemm_gating_refuses_what_the_staged_store_cannot_take(orc):
     gate = dev_as(rng.normal(0, 1, (90, H)), 2)
     with pytest.raises(capi.CaifxError):
         T.qlinear_grouped_forward_swiglu(x, dev(offsets), up_g, gate, 2)
+
+
+@pytest.mark.parametrize("N,K", [(192, 256), (100, 72)])             # matrix-core kernel / shape-agnostic kernel
+def test_grouped_offsets_past_the_buffer_lose_rows_only(orc, N, K):
+    # offsets[E] > total_rows is a caller's mistake; the kernels cut every segment to the buffer instead of
+    # reading and writing past it, so the rows that exist get their expert's result
+    rng = np.random.default_rng(12)
+    total = 100
+    offsets = np.array([0, 60, 160], np.int32)
+    ows, gw = _experts(orc, rng, 2, N, K, "int8pc")
+    x = dev_as(rng.normal(0, 1, (total, K)), 2)
+    dy = dev_as(rng.normal(0, 1e-2, (total, N)), 2)
+    y = host(T.qlinear_grouped_forward(x, dev(offsets), gw, 2))
+    dx = host(T.qlinear_grouped_backward_input(dy, dev(offsets), gw, 2))
+    xh, dyh = host(x), host(dy)
+    for e, (lo, hi) in enumerate(((0, 60), (60, 100))):
+        assert max_rel_err(y[lo:hi], orc.frozen_linear_forward(xh[lo:hi], ows[e], 2)) <= 5e-5
+        assert max_rel_err(dx[lo:hi], orc.frozen_linear_backward(dyh[lo:hi], ows[e], 2)) <= 5e-5
