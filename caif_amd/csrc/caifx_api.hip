@@ -114,6 +114,12 @@ static int forward_impl(int64_t M, int64_t N, int64_t K, const void *x, int x_dt
   // one or two rows: stream each weight row linearly and reduce per row; from three rows on the
   // matrix-core tiling (cost independent of M) is faster; both fall through when a shape does not fit
   st = CAIFX_ERR_UNSUPPORTED;
+  // fp32 compute: beyond a few rows the fp32 matrix-core kernel; up to four rows the VALU decode kernel
+  // below is bound by the weight stream either way
+  if (compute_dtype == CAIFX_F32 && M > 4) {
+    st = mfma_f32_forward(a, s);
+    if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, y, y_dtype, M * N, stream);
+  }
   if (M <= 2) st = rowlin_forward(a, s);
   if (st == CAIFX_ERR_UNSUPPORTED && M <= 16) {
     st = mblock_forward(a, s);
@@ -163,6 +169,10 @@ static int backward_impl(int64_t M, int64_t N, int64_t K, const void *dy, int dy
   GemmArgs a = make_args(M, N, K, dy, dy_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size,
                          dx, dx_dtype, workspace, workspace_bytes);
   hipStream_t s = as_stream(stream);
+  if (compute_dtype == CAIFX_F32) {
+    st = mfma_f32_backward(a, s);
+    if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, dx, dx_dtype, M * K, stream);
+  }
   a.addend = addend;
   st = mfma_backward(a, s);
   if (st != CAIFX_ERR_UNSUPPORTED) return st;         // added in the store
