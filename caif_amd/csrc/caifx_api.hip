@@ -114,9 +114,9 @@ static int forward_impl(int64_t M, int64_t N, int64_t K, const void *x, int x_dt
   // one or two rows: stream each weight row linearly and reduce per row; from three rows on the
   // matrix-core tiling (cost independent of M) is faster; both fall through when a shape does not fit
   st = CAIFX_ERR_UNSUPPORTED;
-  // fp32 compute: beyond a few rows the fp32 matrix-core kernel; up to four rows the VALU decode kernel
-  // below is bound by the weight stream either way
-  if (compute_dtype == CAIFX_F32 && M > 4) {
+  // fp32 compute: from two rows on the fp32 matrix-core kernel (40-43 us at K = N = 4096 whatever M <= 32); the
+  // VALU decode kernel below takes 40-46 us for one row, 49-57 us for two and 66-71 us for four
+  if (compute_dtype == CAIFX_F32 && M > 1) {
     st = mfma_f32_forward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, y, y_dtype, M * N, stream);
   }

@@ -10,13 +10,17 @@
 // matrix cores work on the current one; two barriers per step cost little against the 1000-4000 MFMA
 // cycles between them).  Both operands sit in LDS reduction-major ([r][row] with the row index contiguous),
 // which is what the MFMA operands read: lane (i, h) of a 32x32x2 step takes element [2p + h][i].
+// Up to 32 activation rows a workgroup takes a 32 x 32 tile with 128-deep steps and its four waves split each
+// step's reduction (partial tiles are added through LDS in a fixed order at the end): four times as many
+// workgroups for the same result and a quarter of the barriers.
+#include <type_traits>
+
 #include "caifx_internal.hpp"
 
 namespace caifx {
 namespace {
 
-constexpr int kBK = 32;      // reduction elements per step
-constexpr int kBN = 128;     // result columns per workgroup
+constexpr int kStep = 32;    // the reduction advances in multiples of this (host-side checks, scale-index steps)
 
 struct F32Args {
   int64_t M, N, K;
@@ -26,8 +30,8 @@ struct F32Args {
   const uint8_t *wq;
   const void *scales;
   int group_shift;       // int4: log2(group_size), group_size >= 16
-  int64_t period;        // int8: 0 = no scales, 1 = one scale, otherwise the length of the scale vector (>= 32)
-  uint32_t step;         // int8 scale vector: how far the scale index moves per reduction step, modulo period
+  int64_t period;        // int8: 0 = no scales, 1 = one scale, otherwise the length of the scale vector (>= 32, % 4 == 0)
+  uint32_t step;         // int8 scale vector: how far the scale index moves per 32 reduction elements, modulo period
 };
 
 __device__ __forceinline__ void store_result(void *p, int dt, int64_t i, float v)
@@ -37,28 +41,38 @@ __device__ __forceinline__ void store_result(void *p, int dt, int64_t i, float v
   else static_cast<float *>(p)[i] = v;
 }
 
-// BM = 128: waves 2 x 2 over the tile, 64 x 64 each; BM = 32: waves 1 x 4, 32 x 32 each (small M).
-template <typename XT, bool kInt4, bool kBackward, int BM>
+// Tile shapes (BM x kBN result, kBK deep steps; kBN * kBK = 4096 so that every thread dequantises 16 codes per step):
+//   128 x 128 x 32: waves 2 x 2 over the tile, 64 x 64 each
+//    32 x 128 x 32: waves 1 x 4, 32 x 32 each
+//    32 x  32 x 128: every wave works on the whole tile and takes a quarter of each step's reduction
+// kVec: int8 with a scale vector (length a multiple of 4, 16-byte aligned: four scales per load)
+template <typename XT, bool kInt4, bool kVec, bool kBackward, int BM, int kBN, int kBK>
 __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
 {
+  static_assert(kBN * kBK == 4096, "16 codes per thread and step");
+  constexpr bool kSplit = kBN == 32;       // the waves split the reduction instead of the tile
   constexpr int WM = BM == 128 ? 2 : 1;
-  constexpr int WN = 4 / WM;
+  constexpr int WN = kSplit ? 1 : 4 / WM;
   constexpr int kWaveRows = BM / WM;
   constexpr int kWaveCols = kBN / WN;
   constexpr int TM = kWaveRows / 32;
   constexpr int TN = kWaveCols / 32;
-  constexpr int SA = BM + 4;               // row pitch in floats: the transposing writes spread over the banks
-  constexpr int SB = kBN + 4;
+  // row pitches in floats, chosen so that the transposing writes spread over the banks; the input gradient
+  // writes its weight rows 16 bytes at a time and needs the pitch to keep that alignment
+  constexpr int SA = BM == 32 ? BM + 1 : BM + 4;
+  constexpr int SB = (kBN == 32 && !kBackward) ? kBN + 1 : kBN + 4;
   constexpr int EA = BM * kBK / 256;       // activation elements per thread per step (16 or 4)
   constexpr int TPR = kBK / EA;            // threads per activation row
+  constexpr int kPairs = kSplit ? kBK / 8 : kBK / 2;     // 32x32x2 steps per wave and step
+  static_assert(!kSplit || kBK * SA >= 4 * 16 * 64, "the partial tiles of the four waves fit the activation buffer");
   __shared__ __attribute__((aligned(16))) float As[kBK * SA];
   __shared__ __attribute__((aligned(16))) float Bs[kBK * SB];
 
   const int t = threadIdx.x;
   const int lane = t & 63;
   const int wave = t >> 6;
-  const int wm = wave / WN;
-  const int wn = wave % WN;
+  const int wm = kSplit ? 0 : wave / WN;
+  const int wn = kSplit ? 0 : wave % WN;
   const int64_t R = kBackward ? g.N : g.K;
   const int64_t C = kBackward ? g.K : g.N;
   const int64_t row0 = static_cast<int64_t>(blockIdx.y) * BM;
@@ -71,14 +85,16 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
   int64_t am = row0 + a_row;
   if (am >= g.M) am = g.M - 1;                                   // rows past the end are never stored
   const XT *ap = static_cast<const XT *>(g.a) + am * R + a_col;
-  float areg[EA];
-  auto load_a = [&](int64_t r0) {
+  // two register sets: the loads of steps s+1 and s+2 are in flight while the matrix cores work on step s
+  float areg[2][EA];
+  auto load_a = [&](auto set_, int64_t r0) {
+    constexpr int set = decltype(set_)::value;
     if constexpr (sizeof(XT) == 4) {
 #pragma unroll
       for (int i = 0; i < EA / 4; ++i) {
         const floatx4_t v = *reinterpret_cast<const floatx4_t *>(ap + r0 + 4 * i);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) areg[4 * i + e] = v[e];
+        for (int e = 0; e < 4; ++e) areg[set][4 * i + e] = v[e];
       }
     } else if constexpr (EA == 16) {
 #pragma unroll
@@ -86,25 +102,27 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
         const u32x4_t v = *reinterpret_cast<const u32x4_t *>(ap + r0 + 8 * i);
         const XT *h = reinterpret_cast<const XT *>(&v);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) areg[8 * i + e] = to_f32<XT>(h[e]);
+        for (int e = 0; e < 8; ++e) areg[set][8 * i + e] = to_f32<XT>(h[e]);
       }
     } else {
       const u32x2_t v = *reinterpret_cast<const u32x2_t *>(ap + r0);
       const XT *h = reinterpret_cast<const XT *>(&v);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) areg[e] = to_f32<XT>(h[e]);
+      for (int e = 0; e < 4; ++e) areg[set][e] = to_f32<XT>(h[e]);
     }
   };
-  auto store_a = [&]() {
+  auto store_a = [&](auto set_) {
+    constexpr int set = decltype(set_)::value;
 #pragma unroll
-    for (int e = 0; e < EA; ++e) As[(a_col + e) * SA + a_row] = areg[e];
+    for (int e = 0; e < EA; ++e) As[(a_col + e) * SA + a_row] = areg[set][e];
   };
 
   // ---- weights: 16 consecutive codes (along k) per thread and step
-  //   forward : weight row n = col0 + t/2, k = r0 + (t%2)*16 .. +16      -> Bs[k][n]   (transposing write)
-  //   backward: weight row n = r0 + t/8,   k = col0 + (t%8)*16 .. +16    -> Bs[n][k]   (row write)
-  const int b_major = kBackward ? t >> 3 : t >> 1;
-  const int b_minor = kBackward ? (t & 7) * 16 : (t & 1) * 16;
+  //   forward : weight row n = col0 + t/(kBK/16), k = r0 + (t%(kBK/16))*16 .. +16    -> Bs[k][n]   (transposing write)
+  //   backward: weight row n = r0 + t/(kBN/16),   k = col0 + (t%(kBN/16))*16 .. +16  -> Bs[n][k]   (row write)
+  constexpr int kPerRow = (kBackward ? kBN : kBK) / 16;          // threads per weight row of the piece
+  const int b_major = t / kPerRow;
+  const int b_minor = (t % kPerRow) * 16;
   int64_t flat0;                                                 // flat index n*K + k of the first code at step 0
   if constexpr (!kBackward) {
     int64_t n = col0 + b_major;
@@ -118,42 +136,50 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
   const int64_t flat_step = kBackward ? static_cast<int64_t>(kBK) * g.K : kBK;
   const float *s32 = static_cast<const float *>(g.scales);
   const f16_t *s16 = static_cast<const f16_t *>(g.scales);
-  const bool vec_scales = !kInt4 && g.period > 1;
+  constexpr bool vec_scales = !kInt4 && kVec;
   const uint32_t period = static_cast<uint32_t>(g.period);
   uint32_t sidx = vec_scales ? static_cast<uint32_t>(flat0 % g.period) : 0u;
   const float s_one = (!kInt4 && g.period == 1) ? s32[0] : 1.0f;
 
-  uint32_t wreg[kInt4 ? 2 : 4];
-  float sc[kInt4 ? 1 : 16];
-  auto load_b = [&](int s) {
+  uint32_t wreg[2][kInt4 ? 2 : 4];
+  float sc[2][kInt4 ? 1 : 16];
+  auto load_b = [&](auto set_, int s) {
+    constexpr int set = decltype(set_)::value;
     const int64_t f = flat0 + static_cast<int64_t>(s) * flat_step;
     if constexpr (kInt4) {
       const u32x2_t v = *reinterpret_cast<const u32x2_t *>(g.wq + (f >> 1));
-      wreg[0] = v[0];
-      wreg[1] = v[1];
-      sc[0] = to_f32(s16[f >> g.group_shift]);
+      wreg[set][0] = v[0];
+      wreg[set][1] = v[1];
+      sc[set][0] = to_f32(s16[f >> g.group_shift]);
     } else {
       const u32x4_t v = *reinterpret_cast<const u32x4_t *>(g.wq + f);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) wreg[i] = v[i];
-      if (vec_scales) {
+      for (int i = 0; i < 4; ++i) wreg[set][i] = v[i];
+      if constexpr (vec_scales) {
+        // the first code's flat index is a multiple of 16 and so is every step: quads never straddle the wrap
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          uint32_t idx = sidx + e;
+        for (int q = 0; q < 4; ++q) {
+          uint32_t idx = sidx + 4 * q;
           if (idx >= period) idx -= period;
-          sc[e] = s32[idx];
+          const floatx4_t v4 = *reinterpret_cast<const floatx4_t *>(s32 + idx);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) sc[set][4 * q + e] = v4[e];
         }
-        sidx += g.step;
-        if (sidx >= period) sidx -= period;
+#pragma unroll
+        for (int q = 0; q < kBK / kStep; ++q) {
+          sidx += g.step;
+          if (sidx >= period) sidx -= period;
+        }
       }
     }
   };
-  auto store_b = [&]() {
+  auto store_b = [&](auto set_) {
+    constexpr int set = decltype(set_)::value;
     float w[16];
     if constexpr (kInt4) {
       float e0[8], e1[8];
-      dequant_int4x8(wreg[0], sc[0], e0);
-      dequant_int4x8(wreg[1], sc[0], e1);
+      dequant_int4x8(wreg[set][0], sc[set][0], e0);
+      dequant_int4x8(wreg[set][1], sc[set][0], e1);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         w[e] = e0[e];
@@ -163,9 +189,9 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float q[4];
-        int8x4_to_f32(wreg[i], q);
+        int8x4_to_f32(wreg[set][i], q);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) w[4 * i + e] = vec_scales ? q[e] * sc[4 * i + e] : q[e] * s_one;
+        for (int e = 0; e < 4; ++e) w[4 * i + e] = vec_scales ? q[e] * sc[set][4 * i + e] : q[e] * s_one;
       }
     }
     if constexpr (!kBackward) {
@@ -190,18 +216,20 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
 
   const int li = lane & 31;
   const int lh = lane >> 5;
-  load_a(0);
-  load_b(0);
-  for (int s = 0; s < steps; ++s) {
-    store_a();
-    store_b();
+  typedef std::integral_constant<int, 0> I0;
+  typedef std::integral_constant<int, 1> I1;
+  // No load sits behind a branch (a step past the end re-reads the last one; its registers are never stored),
+  // so the compiler can count the outstanding requests and a wait for one set leaves the other in flight.
+  auto clamped = [&](int s) { return s < steps ? s : steps - 1; };
+  auto one_step = [&](auto set_, int s) {
+    store_a(set_);
+    store_b(set_);
     __syncthreads();
-    if (s + 1 < steps) {          // same for every thread
-      load_a(static_cast<int64_t>(s + 1) * kBK);
-      load_b(s + 1);
-    }
+    load_a(set_, static_cast<int64_t>(clamped(s + 2)) * kBK);
+    load_b(set_, clamped(s + 2));
 #pragma unroll
-    for (int p = 0; p < kBK / 2; ++p) {
+    for (int pp = 0; pp < kPairs; ++pp) {
+      const int p = kSplit ? wave * kPairs + pp : pp;
       const int r = 2 * p + lh;
       float av[TM], bv[TN];
 #pragma unroll
@@ -214,9 +242,41 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
         for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
     }
     __syncthreads();              // the next step overwrites both buffers
+  };
+  load_a(I0{}, 0);
+  load_b(I0{}, 0);
+  load_a(I1{}, static_cast<int64_t>(clamped(1)) * kBK);
+  load_b(I1{}, clamped(1));
+  {
+    int s = 0;
+    for (; s + 2 <= steps; s += 2) {
+      one_step(I0{}, s);
+      one_step(I1{}, s + 1);
+    }
+    if (s < steps) one_step(I0{}, s);
   }
 
   // acc[i][j][r] = D[row][col], row = 8*(r/4) + 4*(lane/32) + r%4, col = lane%32
+  if constexpr (kSplit) {
+    // the loop's last barrier has passed: the activation buffer is free.  Partial tiles [wave][r][lane], then
+    // every thread adds the four partials of four results in wave order.
+#pragma unroll
+    for (int r = 0; r < 16; ++r) As[(wave * 16 + r) * 64 + lane] = acc[0][0][r];
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int o = t + 256 * q;
+      const int r = o >> 6;
+      const int ln = o & 63;
+      float v = As[r * 64 + ln];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) v += As[(w * 16 + r) * 64 + ln];
+      const int64_t row = row0 + 8 * (r >> 2) + 4 * (ln >> 5) + (r & 3);
+      const int64_t col = col0 + (ln & 31);
+      if (row < g.M && col < C) store_result(g.d, g.d_dtype, row * C + col, v);
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -230,22 +290,29 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
     }
 }
 
-template <typename XT, bool kInt4, bool kBackward>
+template <typename XT, bool kInt4, bool kVec, bool kBackward>
 int launch_bm(const F32Args &f, hipStream_t s)
 {
   const int64_t C = kBackward ? f.K : f.N;
-  const int64_t col_tiles = (C + kBN - 1) / kBN;
+  const int64_t R = kBackward ? f.N : f.K;
+  const int64_t col_tiles = (C + 127) / 128;
+  // up to 32 rows: 32-column tiles whose waves split the reduction (128-deep steps)
+  if (f.M <= 32 && R % 128 == 0) {
+    hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 32, 128>), dim3(static_cast<unsigned>((C + 31) / 32), 1), dim3(256), 0,
+                       s, f);
+    return launch_status();
+  }
   // 128-row tiles once there are enough of them to give every compute unit one; below that 32-row tiles
   // put four times as many workgroups on the chip for the same weight traffic through L2
   const int64_t tall = (f.M + 127) / 128;
   if (tall * col_tiles >= 256 && tall <= 65535) {
-    hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kBackward, 128>), dim3(static_cast<unsigned>(col_tiles), static_cast<unsigned>(tall)),
+    hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 128, 128, 32>), dim3(static_cast<unsigned>(col_tiles), static_cast<unsigned>(tall)),
                        dim3(256), 0, s, f);
     return launch_status();
   }
   const int64_t low = (f.M + 31) / 32;
   if (low > 65535) return CAIFX_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kBackward, 32>), dim3(static_cast<unsigned>(col_tiles), static_cast<unsigned>(low)),
+  hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 128, 32>), dim3(static_cast<unsigned>(col_tiles), static_cast<unsigned>(low)),
                      dim3(256), 0, s, f);
   return launch_status();
 }
@@ -253,15 +320,16 @@ int launch_bm(const F32Args &f, hipStream_t s)
 template <typename XT>
 int launch_kind(const F32Args &f, bool int4, bool backward, hipStream_t s)
 {
-  if (int4) return backward ? launch_bm<XT, true, true>(f, s) : launch_bm<XT, true, false>(f, s);
-  return backward ? launch_bm<XT, false, true>(f, s) : launch_bm<XT, false, false>(f, s);
+  if (int4) return backward ? launch_bm<XT, true, false, true>(f, s) : launch_bm<XT, true, false, false>(f, s);
+  if (f.period > 1) return backward ? launch_bm<XT, false, true, true>(f, s) : launch_bm<XT, false, true, false>(f, s);
+  return backward ? launch_bm<XT, false, false, true>(f, s) : launch_bm<XT, false, false, false>(f, s);
 }
 
 int run_f32(const GemmArgs &a, bool backward, hipStream_t s)
 {
   if (a.compute_dtype != CAIFX_F32 || a.offsets || a.addend || a.epilogue) return CAIFX_ERR_UNSUPPORTED;
   const int64_t R = backward ? a.N : a.K;
-  if (R % kBK != 0 || a.K % 32 != 0 || a.K < 32 || a.M < 1 || a.N < 1) return CAIFX_ERR_UNSUPPORTED;
+  if (R % kStep != 0 || a.K % 32 != 0 || a.K < 32 || a.M < 1 || a.N < 1) return CAIFX_ERR_UNSUPPORTED;
   if (a.M > (int64_t{1} << 30) || a.N > (int64_t{1} << 30) || a.K > (int64_t{1} << 30)) return CAIFX_ERR_UNSUPPORTED;
   if (a.N * a.K >= (int64_t{1} << 40)) return CAIFX_ERR_UNSUPPORTED;
   if (!aligned_to(a.x, 16) || !aligned_to(a.w.q, 16)) return CAIFX_ERR_UNSUPPORTED;
@@ -287,9 +355,10 @@ int run_f32(const GemmArgs &a, bool backward, hipStream_t s)
       f.period = 1;
     } else {
       // one conditional subtraction per index: the vector must be at least one step (and one thread's run) long
-      if (a.w.scale_period < 32 || a.w.scale_period > (int64_t{1} << 30) || !aligned_to(a.w.scales, 4)) return CAIFX_ERR_UNSUPPORTED;
+      if (a.w.scale_period < 32 || a.w.scale_period % 4 != 0 || a.w.scale_period > (int64_t{1} << 30) || !aligned_to(a.w.scales, 16))
+        return CAIFX_ERR_UNSUPPORTED;
       f.period = a.w.scale_period;
-      f.step = static_cast<uint32_t>((backward ? static_cast<int64_t>(kBK) * a.K : kBK) % a.w.scale_period);
+      f.step = static_cast<uint32_t>((backward ? static_cast<int64_t>(kStep) * a.K : kStep) % a.w.scale_period);
     }
   } else {
     return CAIFX_ERR_UNSUPPORTED;
