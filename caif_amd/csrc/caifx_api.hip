@@ -126,6 +126,19 @@ static int forward_impl(int64_t M, int64_t N, int64_t K, const void *x, int x_dt
     if (st == CAIFX_ERR_UNSUPPORTED && M <= 4) st = rowlin_forward(a, s);
     if (st == CAIFX_ERR_UNSUPPORTED) st = skinny_forward(a, s);
   }
+  if (M > 16 && M <= 32) {
+    // 17..32 rows: two launches of the 16-row decode kernel (2 x 14-17 us at K = 4096, N = 4096..14336) beat
+    // the tiled GEMM, whose shortest launch is one tile's reduction (43 us int4, 68 us int8 at K = 4096)
+    GemmArgs c = a;
+    c.M = 16;
+    st = mblock_forward(c, s);
+    if (st == CAIFX_OK) {
+      c.M = M - 16;
+      c.x = static_cast<const char *>(x) + 16 * K * static_cast<int64_t>(dtype_size(x_dtype));
+      c.y = static_cast<char *>(y) + 16 * N * static_cast<int64_t>(dtype_size(y_dtype));
+      st = mblock_forward(c, s);
+    }
+  }
   if (st == CAIFX_ERR_UNSUPPORTED) {
     a.addend = addend;
     st = mfma_forward(a, s);

@@ -113,8 +113,10 @@ def test_grouped_equals_per_expert_calls(orc):
     for e in range(E):
         lo, hi = int(offsets[e]), int(offsets[e + 1])
         ye = T.qlinear_forward(x[lo:hi].contiguous(), gw.weights[e], 2, T.BF16)
-        if hi - lo > 16:                                             # same kernel family: bit-identical
+        if hi - lo > 32:                                             # same kernel family: bit-identical
             assert torch.equal(y[lo:hi], ye)
+        else:                                                        # up to 32 rows the plain call takes the decode kernels
+            assert max_rel_err(host(ye), host(y[lo:hi])) <= 8e-3
 
 
 def _route(rng, Tk, top_k, E):

@@ -7,7 +7,7 @@ parity tests normalise.  The asserts are tighter than the contract:
     feed the matrix cores weights that are bit-identical to the oracle's, so only the summation
     order differs (~1e-6);
   * int4 with group size 128 (or a multiple) is scaled after the per-group accumulation, and int8
-    with up to 16 activation rows folds the scales into the activations and multiplies the integer
+    with up to 32 activation rows (two launches of the 16-row kernel from 17 on) folds the scales into the activations and multiplies the integer
     codes exactly on the integer matrix core: both skip the reference's rounding of code*scale to
     the compute dtype; the difference is that rounding, <= 2^-9 per weight with random sign, about
     2e-3 of max|ref| after the sum over K (2e-4 for fp16 compute).
@@ -38,7 +38,7 @@ def _check(orc, rng, M, N, K, kind, cd, xd, group=128, yd=0):
     bound = TOL_32 if cd == 0 else TOL_16
     assert err <= bound, (M, N, K, kind, cd, xd, err)
     if cd != 0 and yd == 0:
-        post = (kind == "int4" and group % 128 == 0) or (kind.startswith("int8") and M <= 16)
+        post = (kind == "int4" and group % 128 == 0) or (kind.startswith("int8") and M <= 32)
         assert err <= (TIGHT_POST if post else TIGHT_16), (M, N, K, kind, cd, xd, err)
     return err
 
@@ -143,3 +143,12 @@ def test_one_hot_reads_a_weight_column_exactly(orc):
                 assert int8_ok(y[0], ow, 5) and int8_ok(y[rows - 1], ow, 900), (kind, N, rows)
                 if rows > 2:
                     assert not y[1:rows - 1].any(), (kind, N, rows)
+
+
+@pytest.mark.parametrize("kind", ["int4", "int8pc", "int8pt"])
+@pytest.mark.parametrize("M", [17, 24, 32])
+def test_two_row_blocks_of_the_decode_kernel(orc, kind, M):
+    # 17..32 rows run as two launches of the 16-row kernel (same accuracy class as M <= 16); row 16 onwards
+    # must come out of the second launch with the right offsets into X and Y
+    _check(orc, np.random.default_rng(700 + M), M, 1536, 1024, kind, 2, 2)
+    _check(orc, np.random.default_rng(701 + M), M, 200, 4096, kind, 1, 1, yd=2)
