@@ -122,7 +122,10 @@ CAIFX_API int caifx_dequantize_int4(const void *packed_data, const void *scales,
  * output type (:442), F16/BF16 fold the caller's following `.To(StorageT)` cast
  * (src/caif_device_moe_frozen_expert.cpp:119-126) into the store and give the
  * same bits as writing fp32 and casting.
- * compute_dtype is the layer's ComputeT.  No dense copy of W is ever written. */
+ * compute_dtype is the layer's ComputeT.  No dense copy of W is ever written.
+ * With up to 32 rows and a 16-bit compute type the memory-bound kernels skip the rounding of code * scale
+ * to the compute type for int8 and for int4 with groups of 128 or more (the products with x are formed
+ * exactly instead): results then differ from the formula above by that rounding, about 2e-3 of max|y|. */
 CAIFX_API int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K,
                           const void *x, int x_dtype, int compute_dtype,
                           const void *wq, int w_kind, const void *scales, int64_t scale_period,
