@@ -13,7 +13,8 @@ not the Python launch path, sets the pace; per-kernel durations for the roofline
 from HIP events around single-kernel graphs on the same stream.
 
 Also reported in `extra`: M in {4,16} decode rates, the cache-resident M=1 rate, the
-compute-bound rows (configs[2..3]) in TFLOP/s and the MoE frozen-expert layer (configs[4]) in tokens/s.
+compute-bound rows (configs[2..3]) in TFLOP/s, the fp32 compute type (configs[0]'s layer) and the MoE
+frozen-expert layer (configs[4]) in tokens/s.
 """
 import argparse
 import json
@@ -26,6 +27,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_FP32_PEAK_TFLOPS = 157.3
 K_DEC, N_DEC = 4096, 14336
 MEASURED_TRAFFIC_INT8_M1 = 59406822     # bytes per launch, rocprofv3 counters (see the roofline object)
 
@@ -267,7 +269,36 @@ def compute_bound_rows(torch, T, dev, gen, capture, time_graph):
             del g
             rows["lora_base_fwd_bwd_M4096_N11008_K4096"] = {
                 "gemm_cast_add_chain_us": round(ms_c * 1e3, 1), "fused_store_us": round(ms_u * 1e3, 1)}
-    return {"prefill_gemm": rows, "moe_frozen_experts": moe_rows(torch, T, dev, gen)}
+    return {"prefill_gemm": rows, "fp32_compute": fp32_rows(torch, T, dev, gen, capture, time_graph),
+            "moe_frozen_experts": moe_rows(torch, T, dev, gen)}
+
+
+def fp32_rows(torch, T, dev, gen, capture, time_graph):
+    """configs[0] on the GPU (int8 per-channel, K = N = 4096, fp32 X[16, 4096], fp32 compute: forward + dX) and
+    the same layer at M = 2048, against the fp32 matrix-core peak."""
+    N = K = 4096
+    w = torch.empty(K, N, device=dev).normal_(0, 0.02, generator=gen)       # the reference's [in,out] labelling
+    q, s = T.quantize_int8(w, per_channel=True)
+    del w
+    fw = T.FrozenWeight(q.reshape(-1), T.W_INT8, s, N, K, N)
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    rows = {}
+    for M, L in ((16, 32), (2048, 8)):
+        x = torch.empty(M, K, device=dev).normal_(0, 1, generator=gen)
+        dy = torch.empty(M, N, device=dev).normal_(0, 1e-3, generator=gen)
+        y, dx = torch.empty(M, N, device=dev), torch.empty(M, K, device=dev)
+        g = capture(lambda i: T.qlinear_forward(x, fw, T.F32, T.F32, out=y, workspace=ws), L)
+        ms_f = time_graph(g, L, reps=3)
+        del g
+        g = capture(lambda i: T.qlinear_backward_input(dy, fw, T.F32, T.F32, out=dx, workspace=ws), L)
+        ms_b = time_graph(g, L, reps=3)
+        del g
+        flops = 2.0 * M * N * K
+        rows[f"int8_M{M}_N{N}_K{K}"] = {
+            "fwd_us": round(ms_f * 1e3, 2), "dx_us": round(ms_b * 1e3, 2),
+            "fwd_TFLOPs": round(flops / (ms_f * 1e-3) / 1e12, 2), "dx_TFLOPs": round(flops / (ms_b * 1e-3) / 1e12, 2),
+            "fwd_dx_frac_of_fp32_mfma_peak": round(2 * flops / ((ms_f + ms_b) * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4)}
+    return rows
 
 
 def moe_rows(torch, T, dev, gen):
