@@ -253,6 +253,10 @@ static int grouped(bool backward, int num_experts, const int32_t *offsets, int64
   a.num_experts = num_experts;
   if (addend && (addend == y || !aligned_to(addend, dtype_size(y_dtype)))) return CAIFX_ERR_INVALID_ARGUMENT;
   hipStream_t s = as_stream(stream);
+  if (compute_dtype == CAIFX_F32 && !addend) {
+    st = backward ? mfma_f32_backward(a, s) : mfma_f32_forward(a, s);
+    if (st != CAIFX_ERR_UNSUPPORTED) return st;
+  }
   a.addend = addend;
   st = backward ? mfma_backward(a, s) : mfma_forward(a, s);
   if (st != CAIFX_ERR_UNSUPPORTED) return st;

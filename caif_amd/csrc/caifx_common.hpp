@@ -112,6 +112,17 @@ __device__ __forceinline__ void int8x4_to_f32(uint32_t p, float (&e)[4])
   e[3] = static_cast<float>(static_cast<int>(p) >> 24);
 }
 
+// Rows [lo, hi) of expert e, forced into 0 <= lo <= hi <= M: offsets that are not non-decreasing or that
+// run past the buffer (a caller's mistake) then lose rows instead of sending loads and stores out of bounds.
+__device__ __forceinline__ void segment_rows(const int32_t *offsets, int e, int64_t M, int &lo, int &hi)
+{
+  const int m = static_cast<int>(M);          // M <= 2^30 is checked on the host
+  lo = offsets[e];
+  hi = offsets[e + 1];
+  lo = lo < 0 ? 0 : (lo > m ? m : lo);
+  hi = hi < lo ? lo : (hi > m ? m : hi);
+}
+
 __device__ __forceinline__ float wave_max(float v)
 {
 #pragma unroll

@@ -96,17 +96,6 @@ template <typename CT> __device__ __forceinline__ uint32_t pack2(float lo, float
   return __builtin_bit_cast(uint32_t, p);
 }
 
-// Rows [lo, hi) of expert e, forced into 0 <= lo <= hi <= M: offsets that are not non-decreasing or that
-// run past the buffer (a caller's mistake) then lose rows instead of sending loads and stores out of bounds.
-__device__ __forceinline__ void segment_rows(const int32_t *offsets, int e, int64_t M, int &lo, int &hi)
-{
-  const int m = static_cast<int>(M);          // M <= 2^30 is checked on the host
-  lo = offsets[e];
-  hi = offsets[e + 1];
-  lo = lo < 0 ? 0 : (lo > m ? m : lo);
-  hi = hi < lo ? lo : (hi > m ? m : hi);
-}
-
 __device__ __forceinline__ float int8_scale_at(const float *scales, int mode, int64_t period, int64_t flat)
 {
   if (mode == SM_SCALAR) return scales ? scales[0] : 1.0f;

@@ -32,6 +32,11 @@ struct F32Args {
   int group_shift;       // int4: log2(group_size), group_size >= 16
   int64_t period;        // int8: 0 = no scales, 1 = one scale, otherwise the length of the scale vector (>= 32, % 4 == 0)
   uint32_t step;         // int8 scale vector: how far the scale index moves per 32 reduction elements, modulo period
+  // grouped form: rows [offsets[e], offsets[e+1]) of a and d belong to expert e and its own weight
+  const int32_t *offsets;
+  const void *const *wq_ptrs;
+  const void *const *scales_ptrs;
+  int num_experts;
 };
 
 __device__ __forceinline__ void store_result(void *p, int dt, int64_t i, float v)
@@ -75,15 +80,35 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
   const int wn = kSplit ? 0 : wave % WN;
   const int64_t R = kBackward ? g.N : g.K;
   const int64_t C = kBackward ? g.K : g.N;
-  const int64_t row0 = static_cast<int64_t>(blockIdx.y) * BM;
+  int64_t row0 = static_cast<int64_t>(blockIdx.y) * BM;
+  int64_t row_hi = g.M;                                          // rows this workgroup may touch end here
   const int64_t col0 = static_cast<int64_t>(blockIdx.x) * kBN;
   const int steps = static_cast<int>(R / kBK);
+  const uint8_t *wq = g.wq;
+  const void *scales = g.scales;
+  if (g.offsets) {
+    // blockIdx.y counts row tiles over all experts (the grid is an upper bound: every expert can add one
+    // partial tile); each thread walks the offsets, which a handful of cache lines hold
+    int tile = blockIdx.y;
+    int e = 0, lo = 0, hi = 0;
+    for (; e < g.num_experts; ++e) {
+      segment_rows(g.offsets, e, g.M, lo, hi);
+      const int tiles = (hi - lo + BM - 1) / BM;
+      if (tile < tiles) break;
+      tile -= tiles;
+    }
+    if (e == g.num_experts) return;                              // the whole workgroup, before any barrier
+    row0 = lo + static_cast<int64_t>(tile) * BM;
+    row_hi = hi;
+    wq = static_cast<const uint8_t *>(g.wq_ptrs[e]);
+    scales = g.scales_ptrs ? g.scales_ptrs[e] : nullptr;
+  }
 
   // ---- activations: thread (a_row, a_col) holds EA consecutive reduction elements of one row
   const int a_row = t / TPR;
   const int a_col = (t % TPR) * EA;
   int64_t am = row0 + a_row;
-  if (am >= g.M) am = g.M - 1;                                   // rows past the end are never stored
+  if (am >= row_hi) am = row_hi - 1;                             // rows past the end are never stored
   const XT *ap = static_cast<const XT *>(g.a) + am * R + a_col;
   // two register sets: the loads of steps s+1 and s+2 are in flight while the matrix cores work on step s
   float areg[2][EA];
@@ -134,8 +159,8 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
     flat0 = static_cast<int64_t>(b_major) * g.K + k;
   }
   const int64_t flat_step = kBackward ? static_cast<int64_t>(kBK) * g.K : kBK;
-  const float *s32 = static_cast<const float *>(g.scales);
-  const f16_t *s16 = static_cast<const f16_t *>(g.scales);
+  const float *s32 = static_cast<const float *>(scales);
+  const f16_t *s16 = static_cast<const f16_t *>(scales);
   constexpr bool vec_scales = !kInt4 && kVec;
   const uint32_t period = static_cast<uint32_t>(g.period);
   uint32_t sidx = vec_scales ? static_cast<uint32_t>(flat0 % g.period) : 0u;
@@ -147,12 +172,12 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
     constexpr int set = decltype(set_)::value;
     const int64_t f = flat0 + static_cast<int64_t>(s) * flat_step;
     if constexpr (kInt4) {
-      const u32x2_t v = *reinterpret_cast<const u32x2_t *>(g.wq + (f >> 1));
+      const u32x2_t v = *reinterpret_cast<const u32x2_t *>(wq + (f >> 1));
       wreg[set][0] = v[0];
       wreg[set][1] = v[1];
       sc[set][0] = to_f32(s16[f >> g.group_shift]);
     } else {
-      const u32x4_t v = *reinterpret_cast<const u32x4_t *>(g.wq + f);
+      const u32x4_t v = *reinterpret_cast<const u32x4_t *>(wq + f);
 #pragma unroll
       for (int i = 0; i < 4; ++i) wreg[set][i] = v[i];
       if constexpr (vec_scales) {
@@ -273,7 +298,7 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
       for (int w = 1; w < 4; ++w) v += As[(w * 16 + r) * 64 + ln];
       const int64_t row = row0 + 8 * (r >> 2) + 4 * (ln >> 5) + (r & 3);
       const int64_t col = col0 + (ln & 31);
-      if (row < g.M && col < C) store_result(g.d, g.d_dtype, row * C + col, v);
+      if (row < row_hi && col < C) store_result(g.d, g.d_dtype, row * C + col, v);
     }
     return;
   }
@@ -285,7 +310,7 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int64_t row = row0 + wm * kWaveRows + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-        if (row < g.M && col < C) store_result(g.d, g.d_dtype, row * C + col, acc[i][j][r]);
+        if (row < row_hi && col < C) store_result(g.d, g.d_dtype, row * C + col, acc[i][j][r]);
       }
     }
 }
@@ -296,6 +321,17 @@ int launch_bm(const F32Args &f, hipStream_t s)
   const int64_t C = kBackward ? f.K : f.N;
   const int64_t R = kBackward ? f.N : f.K;
   const int64_t col_tiles = (C + 127) / 128;
+  if (f.offsets) {
+    // segment lengths live on the device; the host knows their mean: 128-row tiles when an expert has that
+    // many rows on average, 32-row tiles otherwise; every expert can add one partial tile
+    const bool tall_tiles = f.M >= static_cast<int64_t>(f.num_experts) * 128;
+    const int64_t row_tiles = (f.M + (tall_tiles ? 127 : 31)) / (tall_tiles ? 128 : 32) + f.num_experts;
+    if (row_tiles > 65535) return CAIFX_ERR_UNSUPPORTED;
+    const dim3 grid(static_cast<unsigned>(col_tiles), static_cast<unsigned>(row_tiles));
+    if (tall_tiles) hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 128, 128, 32>), grid, dim3(256), 0, s, f);
+    else hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 128, 32>), grid, dim3(256), 0, s, f);
+    return launch_status();
+  }
   // up to 32 rows: 32-column tiles whose waves split the reduction (128-deep steps)
   if (f.M <= 32 && R % 128 == 0) {
     hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 32, 128>), dim3(static_cast<unsigned>((C + 31) / 32), 1), dim3(256), 0,
@@ -327,12 +363,14 @@ int launch_kind(const F32Args &f, bool int4, bool backward, hipStream_t s)
 
 int run_f32(const GemmArgs &a, bool backward, hipStream_t s)
 {
-  if (a.compute_dtype != CAIFX_F32 || a.offsets || a.addend || a.epilogue) return CAIFX_ERR_UNSUPPORTED;
+  if (a.compute_dtype != CAIFX_F32 || a.addend || a.epilogue) return CAIFX_ERR_UNSUPPORTED;
+  const bool grouped = a.offsets != nullptr;
+  if (grouped && (a.num_experts < 1 || !a.wq_ptrs)) return CAIFX_ERR_UNSUPPORTED;
   const int64_t R = backward ? a.N : a.K;
   if (R % kStep != 0 || a.K % 32 != 0 || a.K < 32 || a.M < 1 || a.N < 1) return CAIFX_ERR_UNSUPPORTED;
   if (a.M > (int64_t{1} << 30) || a.N > (int64_t{1} << 30) || a.K > (int64_t{1} << 30)) return CAIFX_ERR_UNSUPPORTED;
   if (a.N * a.K >= (int64_t{1} << 40)) return CAIFX_ERR_UNSUPPORTED;
-  if (!aligned_to(a.x, 16) || !aligned_to(a.w.q, 16)) return CAIFX_ERR_UNSUPPORTED;
+  if (!aligned_to(a.x, 16) || (!grouped && !aligned_to(a.w.q, 16))) return CAIFX_ERR_UNSUPPORTED;
   const bool int4 = a.w.kind == CAIFX_W_INT4_GROUP;
 
   F32Args f{};
@@ -344,18 +382,24 @@ int run_f32(const GemmArgs &a, bool backward, hipStream_t s)
   f.d_dtype = a.y_dtype;
   f.wq = static_cast<const uint8_t *>(a.w.q);
   f.scales = a.w.scales;
+  f.offsets = a.offsets;
+  f.wq_ptrs = a.wq_ptrs;
+  f.scales_ptrs = a.scales_ptrs;
+  f.num_experts = a.num_experts;
+  // grouped: the per-expert pointers live on the device; one allocation per expert keeps them 16-byte aligned
+  const bool has_scales = grouped ? a.scales_ptrs != nullptr : a.w.scales != nullptr;
   if (int4) {
     const int gs = a.w.group_size;
-    if (!a.w.scales || gs < 16 || (gs & (gs - 1)) != 0) return CAIFX_ERR_UNSUPPORTED;   // 16 codes of a thread share a scale
+    if (!has_scales || gs < 16 || (gs & (gs - 1)) != 0) return CAIFX_ERR_UNSUPPORTED;   // 16 codes of a thread share a scale
     f.group_shift = __builtin_ctz(static_cast<unsigned>(gs));
   } else if (a.w.kind == CAIFX_W_INT8) {
-    if (!a.w.scales) {
+    if (!has_scales) {
       f.period = 0;
     } else if (a.w.scale_period == 1) {
       f.period = 1;
     } else {
       // one conditional subtraction per index: the vector must be at least one step (and one thread's run) long
-      if (a.w.scale_period < 32 || a.w.scale_period % 4 != 0 || a.w.scale_period > (int64_t{1} << 30) || !aligned_to(a.w.scales, 16))
+      if (a.w.scale_period < 32 || a.w.scale_period % 4 != 0 || a.w.scale_period > (int64_t{1} << 30) || (!grouped && !aligned_to(a.w.scales, 16)))
         return CAIFX_ERR_UNSUPPORTED;
       f.period = a.w.scale_period;
       f.step = static_cast<uint32_t>((backward ? static_cast<int64_t>(kStep) * a.K : kStep) % a.w.scale_period);

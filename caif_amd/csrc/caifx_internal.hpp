@@ -55,8 +55,8 @@ int mfma_forward(const GemmArgs &a, hipStream_t s);
 int mfma_backward(const GemmArgs &a, hipStream_t s);
 size_t mfma_workspace_bytes(const GemmArgs &a, bool backward);
 
-// fp32 compute type on the matrix cores (v_mfma_f32_32x32x2_f32), forward and input gradient, any M.
-// CAIFX_ERR_UNSUPPORTED for grouped problems, an addend, reductions that are not a multiple of 32,
+// fp32 compute type on the matrix cores (v_mfma_f32_32x32x2_f32), forward and input gradient, any M, plain
+// and grouped.  CAIFX_ERR_UNSUPPORTED for an addend, reductions that are not a multiple of 32,
 // int4 groups below 16 or not a power of two, int8 scale vectors shorter than 32 or not a multiple of 4 long.
 int mfma_f32_forward(const GemmArgs &a, hipStream_t s);
 int mfma_f32_backward(const GemmArgs &a, hipStream_t s);

@@ -24,7 +24,7 @@ def test_fp32_compute_forward_and_input_gradient(orc, kind, group, M, N, K):
     if kind == "int4" and (N * K) % group:
         pytest.skip("whole groups only")
     ow, dw = make_weight(orc, rng, N, K, kind, group, std=0.02 if kind != "int8raw" else 1.0)
-    for xdt in (0, 2):
+    for xdt in (0, 2, 1):
         x = dev_as(rng.normal(0, 1, (M, K)), xdt)
         dy = dev_as(rng.normal(0, 1e-3, (M, N)), xdt)
         y = host(T.qlinear_forward(x, dw, T.F32))
@@ -76,3 +76,34 @@ def test_fp32_compute_config0_shape_and_large_m(orc):
     yb = T.qlinear_forward(xb, dw, T.F32, y_dtype=T.BF16)
     import torch
     assert torch.equal(yb[rows], T.qlinear_forward(xb, dw, T.F32)[rows].to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("kind,group", [("int8pc", 128), ("int8pt", 128), ("int4", 32)])
+@pytest.mark.parametrize("counts", [[130, 0, 1, 257, 64, 5],        # mean below 128 rows: 32-row tiles
+                                    [300, 129, 0, 256, 128, 200]])  # mean above: 128-row tiles, partial last tiles
+def test_fp32_compute_grouped_segments(orc, kind, group, counts):
+    # the MoE wrapper's ComputeT = float cells: expert segments on the fp32 matrix-core kernel; rows past the
+    # last segment are not written
+    from gpu_helpers import dev
+    from caif_amd import torch_ops as TT
+    import torch
+    rng = np.random.default_rng(sum(counts) + group)
+    E, N, K = len(counts), 192, 256
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    total = int(offsets[-1])
+    pairs = [make_weight(orc, rng, N, K, kind, group) for _ in range(E)]
+    gw = TT.GroupedFrozenWeights([p[1] for p in pairs])
+    x = dev_as(rng.normal(0, 1, (total + 3, K)), 0)
+    dy = dev_as(rng.normal(0, 1e-2, (total + 3, N)), 0)
+    y = torch.full((total + 3, N), 7.0, device="cuda")
+    dx = torch.full((total + 3, K), 5.0, device="cuda")
+    TT.qlinear_grouped_forward(x, dev(offsets), gw, TT.F32, TT.F32, out=y)
+    TT.qlinear_grouped_backward_input(dy, dev(offsets), gw, TT.F32, TT.F32, out=dx)
+    yh, dxh, xh, dyh = host(y), host(dx), host(x), host(dy)
+    for e in range(E):
+        lo, hi = offsets[e], offsets[e + 1]
+        if hi == lo:
+            continue
+        assert max_rel_err(yh[lo:hi], orc.frozen_linear_forward(xh[lo:hi], pairs[e][0], orc.F32)) <= TOL, (kind, e)
+        assert max_rel_err(dxh[lo:hi], orc.frozen_linear_backward(dyh[lo:hi], pairs[e][0], orc.F32)) <= TOL, (kind, e)
+    assert np.all(yh[total:] == 7.0) and np.all(dxh[total:] == 5.0)
