@@ -1,0 +1,62 @@
+"""GPU parity at the largest sizes: a weight of more than 2^31 elements (N = 270336, K = 8192), so that every
+kernel's flat index n*K + k, byte offsets and scale indices pass 2^31 on the high rows.  The CPU oracle would need
+minutes and tens of GB for this, so the check is a size-independent property: the last rows of the big weight,
+taken as a weight of their own, give the reference (torch fp32 matmul on the dequantised slice; int8 codes and
+int4 code * scale products are formed independently of the library with torch ops)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from caif_amd import torch_ops as T                                  # noqa: E402
+
+N, K, R = 270336, 8192, 4096           # N*K = 2.2e9 > 2^31; R = rows checked at the top end
+
+
+def _rel(got, want):
+    return float((got.double() - want.double()).abs().max() / want.double().abs().max())
+
+
+def _int8_weight(gen, scale):
+    q = torch.randint(-127, 128, (N * K,), device="cuda", dtype=torch.int8, generator=gen)
+    s = torch.tensor([scale], device="cuda") if scale else None
+    dense_top = q[-R * K:].view(R, K).float() * (scale if scale else 1.0)
+    return T.FrozenWeight(q, T.W_INT8, s, N, K, 1), dense_top
+
+
+def _int4_weight(gen):
+    p = torch.randint(0, 256, (N * K // 2,), device="cuda", dtype=torch.uint8, generator=gen)
+    s = (torch.rand(N * K // 128, device="cuda", generator=gen) * 0.01 + 0.001).to(torch.float16)
+    pt = p[-R * K // 2:].to(torch.int16)
+    lo, hi = pt & 15, pt >> 4
+    codes = torch.stack([lo, hi], dim=1).reshape(-1)
+    codes = torch.where(codes >= 8, codes - 16, codes).float()
+    dense_top = (codes * s[-R * K // 128:].float().repeat_interleave(128)).view(R, K)
+    return T.FrozenWeight(p, T.W_INT4_GROUP, s, N, K, 1, 128), dense_top
+
+
+@pytest.mark.parametrize("kind", ["int8raw", "int8pt", "int4"])
+def test_flat_indices_beyond_2_31(kind):
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    fw, dense_top = _int4_weight(gen) if kind == "int4" else _int8_weight(gen, 0.0 if kind == "int8raw" else 0.0123)
+    w_bf16 = dense_top.to(torch.bfloat16).float()                  # what the reference feeds its GEMM
+    for M in (1, 2, 16, 24, 64):                                    # row-streaming, row-block, two row blocks, tiled GEMM
+        x = torch.randn(M, K, device="cuda", generator=gen).to(torch.bfloat16)
+        y = T.qlinear_forward(x, fw, T.BF16)
+        want = x.float() @ w_bf16.t()
+        # up to 32 rows the kernels skip the bf16 rounding of code*scale (exact for bare int8 codes)
+        tol = 2e-5 if (M > 32 or kind == "int8raw") else 4e-3
+        assert _rel(y[:, -R:], want) <= tol, (kind, M)
+    # input gradient: dY is zero outside the top rows, so only they contribute, but every row is visited
+    for M in (8, 64):
+        dy = torch.zeros(M, N, device="cuda", dtype=torch.bfloat16)
+        dy[:, -R:] = torch.randn(M, R, device="cuda", generator=gen).to(torch.bfloat16)
+        dx = T.qlinear_backward_input(dy, fw, T.BF16)
+        assert _rel(dx, dy[:, -R:].float() @ w_bf16) <= 2e-5, (kind, M)
+    # fp32 compute type on the same weight
+    x = torch.randn(16, K, device="cuda", generator=gen)
+    assert _rel(T.qlinear_forward(x, fw, T.F32)[:, -R:], x @ dense_top.t()) <= 1e-4, kind
+    dy = torch.zeros(40, N, device="cuda")
+    dy[:, -R:] = torch.randn(40, R, device="cuda", generator=gen)
+    assert _rel(T.qlinear_backward_input(dy, fw, T.F32), dy[:, -R:] @ dense_top) <= 1e-4, kind
