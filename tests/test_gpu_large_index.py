@@ -60,3 +60,48 @@ def test_flat_indices_beyond_2_31(kind):
     dy = torch.zeros(40, N, device="cuda")
     dy[:, -R:] = torch.randn(40, R, device="cuda", generator=gen)
     assert _rel(T.qlinear_backward_input(dy, fw, T.F32), dy[:, -R:] @ dense_top) <= 1e-4, kind
+
+
+def test_quantisers_beyond_2_31_elements():
+    # codes and scales of 2^31 + 2^21 elements against the reference's arithmetic restated with torch ops
+    # (IEEE fp32 division for max/127, max/7 and 1/scale, one rounding for x * inv, clamp, round half to even;
+    # src/caif_cuda_kernels_quant.cu:258-362,384-444,502-559); bit-exact, as at the small sizes the oracle covers
+    rows, cols = 262400, 8192
+    n = rows * cols
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(9)
+    x = torch.randn(n, device="cuda", generator=gen)
+    x[-5] = 7.5                                                      # the maximum sits beyond 2^31
+    # torch divides by a Python scalar through its reciprocal; tensor / tensor is the IEEE division the kernels use
+    c127, c7, one = (torch.tensor(v, device="cuda") for v in (127.0, 7.0, 1.0))
+    # per tensor
+    q, s = T.quantize_int8(x, per_channel=False)
+    scale = x.abs().max() / c127
+    assert torch.equal(s, scale.reshape(1))
+    want = (x * (one / scale)).clamp_(-127.0, 127.0).round_().to(torch.int8)
+    assert torch.equal(q, want)
+    del q, want
+    # per channel: scale[c] over the rows of column c
+    x2 = x.view(rows, cols)
+    q, s = T.quantize_int8(x2, per_channel=True)
+    scale = x2.abs().amax(dim=0) / c127
+    assert torch.equal(s, scale)
+    want = (x2 * (one / scale)).clamp_(-127.0, 127.0).round_().to(torch.int8)
+    assert torch.equal(q, want)
+    back = T.dequantize_int8(q, s, per_channel=True)
+    assert torch.equal(back, q.float() * s)
+    del q, want, back
+    # int4, groups of 128 along the flat index
+    p, s16 = T.quantize_int4_per_group(x, 128)
+    g = x.view(-1, 128)
+    s32 = g.abs().amax(dim=1) / c7
+    assert torch.equal(s16, s32.to(torch.float16))
+    codes = (g * (one / s32).unsqueeze(1)).clamp_(-7.0, 7.0).round_().to(torch.int16).view(-1) & 15
+    want = (codes[0::2] | (codes[1::2] << 4)).to(torch.uint8)
+    assert torch.equal(p, want)
+    del codes, want, g
+    back = T.dequantize_int4_per_group(p, s16, n, 128)
+    lo, hi = (p & 15).to(torch.int16), (p >> 4).to(torch.int16)
+    c = torch.stack([lo, hi], dim=1).reshape(-1)
+    c = torch.where(c >= 8, c - 16, c).float()
+    assert torch.equal(back, c * s16.float().repeat_interleave(128))
