@@ -1,0 +1,93 @@
+"""The library's launches recorded into a HIP graph (callers such as the bench replay them; the launchers clear
+their accumulators with fill kernels, never with memset nodes): every replay must return what the same calls
+return eagerly on the inputs the buffers hold at that moment.  The graph is replayed several times with new
+inputs and eager work and synchronisations in between, and every replay is compared bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from caif_amd import torch_ops as T                                  # noqa: E402
+
+
+def test_replays_equal_eager_results():
+    dev = torch.device("cuda")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(3)
+    N, K, E, Tk, top_k, D = 512, 1024, 4, 96, 2, 256
+    w = torch.empty(K, N, device=dev).normal_(0, 0.02, generator=gen)
+    q8, s8 = T.quantize_int8(w, per_channel=True)
+    fw8 = T.FrozenWeight(q8.reshape(-1), T.W_INT8, s8, N, K, N)
+    p4, s4 = T.quantize_int4_per_group(w.reshape(N, K), 128)
+    fw4 = T.FrozenWeight(p4, T.W_INT4_GROUP, s4, N, K, 1, 128)
+    experts = []
+    for _ in range(E):
+        we = torch.empty(D, D, device=dev).normal_(0, 0.02, generator=gen)
+        qe, se = T.quantize_int8(we, per_channel=True)
+        experts.append(T.FrozenWeight(qe.reshape(-1), T.W_INT8, se, D, D, D))
+    gw = T.GroupedFrozenWeights(experts)
+
+    # static inputs, refilled before every replay
+    wsrc = torch.empty(K, N, device=dev)
+    x1, x16, x64 = (torch.empty(m, K, device=dev, dtype=torch.bfloat16) for m in (1, 16, 64))
+    dy64 = torch.empty(64, N, device=dev, dtype=torch.bfloat16)
+    xf = torch.empty(16, K, device=dev)
+    tok = torch.empty(Tk, D, device=dev, dtype=torch.bfloat16)
+    idx = torch.empty(Tk, top_k, device=dev, dtype=torch.int32)
+    wts = torch.empty(Tk, top_k, device=dev, dtype=torch.bfloat16)
+    rows = Tk * top_k
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+
+    def refill(seed):
+        g = torch.Generator(device=dev)
+        g.manual_seed(seed)
+        wsrc.normal_(0, 0.02, generator=g)
+        for t in (x1, x16, x64, tok):
+            t.copy_(torch.empty(t.shape, device=dev).normal_(0, 1, generator=g))
+        dy64.copy_(torch.empty(64, N, device=dev).normal_(0, 1e-2, generator=g))
+        xf.normal_(0, 1, generator=g)
+        idx.copy_(torch.randint(0, E, (Tk, top_k), device=dev, generator=g).to(torch.int32))
+        wts.copy_(torch.softmax(torch.empty(Tk, top_k, device=dev).normal_(0, 1, generator=g), dim=1))
+
+    def work():
+        out = {}
+        out["q8"], out["s8"] = T.quantize_int8(wsrc, per_channel=True)          # column maxima through atomics
+        out["qt"], out["st"] = T.quantize_int8(wsrc, per_channel=False)
+        out["p4"], out["s4"] = T.quantize_int4_per_group(wsrc, 128)
+        out["y1_4"] = T.qlinear_forward(x1, fw4, T.BF16, workspace=ws)
+        out["y1_8"] = T.qlinear_forward(x1, fw8, T.BF16, workspace=ws)
+        out["y16"] = T.qlinear_forward(x16, fw8, T.BF16, workspace=ws)
+        out["y64"] = T.qlinear_forward(x64, fw4, T.BF16, workspace=ws)
+        out["dx64"] = T.qlinear_backward_input(dy64, fw8, T.BF16, workspace=ws)
+        out["yf"] = T.qlinear_forward(xf, fw8, T.F32, workspace=ws)
+        dmap, offs = T.moe_build_dispatch_map(idx, E)                            # counters, scans
+        packed = T.moe_dispatch(tok, idx, dmap, offs, rows, out=torch.empty(rows, D, device=dev, dtype=torch.bfloat16))
+        ye = T.qlinear_grouped_forward(packed, offs, gw, T.BF16, T.BF16, workspace=ws,
+                                       out=torch.empty(rows, D, device=dev, dtype=torch.bfloat16))
+        out["dmap"], out["offs"], out["packed"], out["ye"] = dmap, offs, packed, ye
+        out["comb"] = T.moe_combine(ye, idx, wts, dmap, offs)
+        return out
+
+    refill(100)
+    work()                                                           # warm up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            captured = work()
+    torch.cuda.synchronize()
+
+    for rep in range(4):
+        refill(200 + rep)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = {k: v.clone() for k, v in captured.items()}
+        want = work()                                                # the program's own eager work between replays
+        torch.cuda.synchronize()
+        for k in want:
+            assert torch.equal(got[k], want[k]), (rep, k)
+    assert not np.isnan(got["comb"].float().cpu().numpy()).any()
