@@ -80,6 +80,10 @@ struct TileArgs {
   const void *const *wq_ptrs;
   const void *const *scales_ptrs;
   int num_experts;
+  // plain form with few tiles: ksplit workgroups share a tile, each takes split_steps 64-deep steps of the
+  // reduction and writes its fp32 partial tile to d + split * M * C (d is then the caller's workspace)
+  int ksplit;
+  int split_steps;
 };
 
 // byte offset of 16-byte chunk `chunk` (0..7) of LDS tile row `row`.  The chunk position is XORed
@@ -134,6 +138,7 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
 
   // ---- which tile -----------------------------------------------------------------------
   int64_t row_lo, row_hi;        // rows of A / D this workgroup may touch: [row_lo, row_hi)
+  int split = 0;                 // which part of the reduction (plain form with ksplit > 1)
   int64_t col_tile = blockIdx.x;
   const uint8_t *wq = static_cast<const uint8_t *>(g.wq);
   const void *scales = g.scales;
@@ -206,8 +211,10 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
     constexpr int kBandTiles = 512 / BM;
     const int64_t col_tiles = (C + BC - 1) / BC;
     const int64_t row_tiles = (g.M + BM - 1) / BM;
-    const int64_t per_xcd = gridDim.x >> 3;
-    const int64_t pos = static_cast<int64_t>(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    const unsigned bid = blockIdx.x / static_cast<unsigned>(g.ksplit);
+    split = static_cast<int>(blockIdx.x - bid * static_cast<unsigned>(g.ksplit));
+    const int64_t per_xcd = (gridDim.x / static_cast<unsigned>(g.ksplit)) >> 3;
+    const int64_t pos = static_cast<int64_t>(bid & 7) * per_xcd + (bid >> 3);
     if (pos >= row_tiles * col_tiles) return;
     const int64_t band = pos / (kBandTiles * col_tiles);
     const int64_t within = pos - band * kBandTiles * col_tiles;
@@ -289,7 +296,7 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
   //   backward int8: same rows, 8 codes (8 B)
   uint32_t wreg[2][8];
   f16_t wscale[2][4];
-  int64_t w_flat[4];       // flat index n*K + k of each register row's first code at step 0
+  int64_t w_flat[4] = {0, 0, 0, 0};   // flat index n*K + k of each register row's first code at step 0
   const f16_t *s16 = static_cast<const f16_t *>(scales);
   const float *s32 = static_cast<const float *>(scales);
   int wf_c = 0, wf_r = 0;  // forward: tile-local column / first r;  backward: first r row / first c
@@ -324,13 +331,25 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
   floatx4_t wsc8[2][8];
   uint32_t sidx[4] = {0, 0, 0, 0};
   const uint32_t period32 = static_cast<uint32_t>(g.period);
+  int steps = static_cast<int>(R / BR);
+  if constexpr (!kGrouped) {
+    if (g.ksplit > 1) {
+      // this workgroup's part of the reduction: everything below counts steps from its first one
+      const int first = split * g.split_steps;
+      const int64_t r_begin = static_cast<int64_t>(first) * BR;
+      steps = steps - first < g.split_steps ? steps - first : g.split_steps;
+#pragma unroll
+      for (int i = 0; i < kAChunks; ++i) a_ptr[i] += r_begin;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w_flat[i] += kBackward ? r_begin * g.K : r_begin;
+    }
+  }
   if constexpr (!kInt4) {
     if (g.scale_mode == SM_VEC4) {
 #pragma unroll
       for (int i = 0; i < (kBackward ? 4 : 2); ++i) sidx[i] = static_cast<uint32_t>(w_flat[i] % g.period);
     }
   }
-  const int steps = static_cast<int>(R / BR);
   const int last = steps - 1;
   auto tile_r0 = [&](int t) { return static_cast<int64_t>(t < last ? t : last) * BR; };   // clamped: reloading the last tile is harmless
   auto load_w = [&](auto set_, int t) {
@@ -572,6 +591,7 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
   }
 
   // ---- epilogue: acc[i][j][r] = D[row][col], row = 8*(r/4) + 4*(lane/32) + r%4, col = lane%32
+  const int64_t d_off = static_cast<int64_t>(split) * g.M * C;      // partial tiles of a shared reduction: one [M, C] slab per part
   // A lane's values sit in 16 different rows, one element each, so a direct store moves 64- or 128-byte pieces
   // with one instruction per element.  After the last barrier nobody reads the operand tiles any more, so each
   // consumer wave lays its (BM/2) x 64 sub-tile out in a private piece of LDS (row pitch = row + 16 bytes:
@@ -610,7 +630,7 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
           const int64_t grow = row_lo + wm * kWaveRows + pass * kRowsPerPass + lrow;
           if (grow < row_hi && gcol < C) {
             u32x4_t v = *reinterpret_cast<const u32x4_t *>(stage + lrow * kPitch + chunk * 16);
-            const int64_t o = grow * C + gcol;
+            const int64_t o = d_off + grow * C + gcol;
             if constexpr (sizeof(T) == 2 && kGrouped) {        // only the grouped launches carry these
               if (g.epilogue != EPI_NONE) {
                 const u32x4_t gv = *reinterpret_cast<const u32x4_t *>(static_cast<const T *>(g.e1) + o);
@@ -663,7 +683,7 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
         for (int r = 0; r < 16; ++r) {
           const int64_t row = row_lo + wm * kWaveRows + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
           if (row < row_hi) {
-            const int64_t o = row * C + col;
+            const int64_t o = d_off + row * C + col;
             float v = acc[i][j][r];
             if (g.addend) {
               // the caller's cast of this result to the tensor dtype followed by an element-wise Add, same roundings
@@ -704,7 +724,7 @@ int launch_one(const TileArgs &t, int64_t row_tiles, hipStream_t s)
   const int64_t col_tiles = (C + BC - 1) / BC;
   dim3 grid(static_cast<unsigned>(col_tiles), static_cast<unsigned>(row_tiles));
   {
-    const int64_t padded = (row_tiles * col_tiles + 7) / 8 * 8;      // linear grid, see the tile numbering in the kernel
+    const int64_t padded = (row_tiles * col_tiles + 7) / 8 * 8 * (kGrouped ? 1 : t.ksplit);      // linear grid, see the tile numbering in the kernel
     if (padded > 0x7fffffff) return CAIFX_ERR_UNSUPPORTED;
     grid = dim3(static_cast<unsigned>(padded), 1);
   }
@@ -762,6 +782,48 @@ int pick_kind(const TileArgs &t, bool int4, bool backward, bool grouped, hipStre
 {
   if (int4) return backward ? launch_tile<CT, XT, true, true>(t, grouped, s) : launch_tile<CT, XT, true, false>(t, grouped, s);
   return backward ? launch_tile<CT, XT, false, true>(t, grouped, s) : launch_tile<CT, XT, false, false>(t, grouped, s);
+}
+
+// y[i] = T(sum over the parts of partial[part][i]) in part order, then the optional addend with the roundings
+// of the cast and the Add
+template <typename T>
+__global__ void splitk_reduce_kernel(const float *__restrict__ partial, int parts, int64_t n, T *__restrict__ y,
+                                     const T *__restrict__ addend)
+{
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float v = partial[i];
+  for (int p = 1; p < parts; ++p) v += partial[p * n + i];
+  if (addend) v = round_through<T>(v) + to_f32<T>(addend[i]);
+  y[i] = from_f32<T>(v);
+}
+
+// With fewer tiles than compute units the launch lasts one tile's whole reduction (43-70 us at K = 4096) however
+// few rows there are.  Then up to 8 workgroups share a tile's reduction, each at least 8 steps of it, and write
+// fp32 partial tiles to the caller's workspace; a second launch adds them in a fixed order.
+struct SplitPlan {
+  int ksplit;
+  int split_steps;
+  size_t bytes;
+};
+SplitPlan plan_split(int64_t M, int64_t C, int64_t R, bool grouped)
+{
+  SplitPlan p{1, 0, 0};
+  if (grouped || R % BR != 0) return p;
+  const int64_t tiles = ((M + 127) / 128) * ((C + BC - 1) / BC);
+  const int64_t steps = R / BR;
+  if (tiles > 96 || steps < 16) return p;
+  int64_t k = 256 / tiles;
+  if (k > 8) k = 8;
+  if (k > steps / 8) k = steps / 8;
+  if (k < 2) return p;
+  const int64_t per = (steps + k - 1) / k;
+  k = (steps + per - 1) / per;                   // every part has at least one step
+  if (k < 2) return p;
+  p.ksplit = static_cast<int>(k);
+  p.split_steps = static_cast<int>(per);
+  p.bytes = static_cast<size_t>(k) * static_cast<size_t>(M) * static_cast<size_t>(C) * sizeof(float);
+  return p;
 }
 
 int run(const GemmArgs &a, bool backward, hipStream_t s)
@@ -822,18 +884,49 @@ int run(const GemmArgs &a, bool backward, hipStream_t s)
       t.scale_mode = SM_ANY;
     }
   }
-  if (a.compute_dtype == CAIFX_BF16) {
-    if (a.x_dtype == CAIFX_F32) return pick_kind<bf16_t, float>(t, int4, backward, grouped, s);
-    return pick_kind<bf16_t, bf16_t>(t, int4, backward, grouped, s);
+  t.ksplit = 1;
+  const int64_t cols = backward ? a.K : a.N;
+  const SplitPlan plan = plan_split(a.M, cols, R, grouped);
+  const bool split = plan.ksplit > 1 && a.epilogue == EPI_NONE && a.workspace && a.workspace_bytes >= plan.bytes &&
+                     aligned_to(a.workspace, 16);
+  if (split) {
+    t.ksplit = plan.ksplit;
+    t.split_steps = plan.split_steps;
+    t.d = a.workspace;
+    t.d_dtype = CAIFX_F32;
+    t.addend = nullptr;
+    t.vec_store = cols % 8 == 0;
   }
-  if (a.x_dtype == CAIFX_F32) return pick_kind<f16_t, float>(t, int4, backward, grouped, s);
-  return pick_kind<f16_t, f16_t>(t, int4, backward, grouped, s);
+  int st;
+  if (a.compute_dtype == CAIFX_BF16) {
+    st = a.x_dtype == CAIFX_F32 ? pick_kind<bf16_t, float>(t, int4, backward, grouped, s) : pick_kind<bf16_t, bf16_t>(t, int4, backward, grouped, s);
+  } else {
+    st = a.x_dtype == CAIFX_F32 ? pick_kind<f16_t, float>(t, int4, backward, grouped, s) : pick_kind<f16_t, f16_t>(t, int4, backward, grouped, s);
+  }
+  if (!split || st != CAIFX_OK) return st;
+  const int64_t n = a.M * cols;
+  const dim3 grid(static_cast<unsigned>((n + 255) / 256));
+  const float *partial = static_cast<const float *>(a.workspace);
+  if (a.y_dtype == CAIFX_F32)
+    hipLaunchKernelGGL(splitk_reduce_kernel<float>, grid, dim3(256), 0, s, partial, plan.ksplit, n, static_cast<float *>(a.y),
+                       static_cast<const float *>(a.addend));
+  else if (a.y_dtype == CAIFX_BF16)
+    hipLaunchKernelGGL(splitk_reduce_kernel<bf16_t>, grid, dim3(256), 0, s, partial, plan.ksplit, n, static_cast<bf16_t *>(a.y),
+                       static_cast<const bf16_t *>(a.addend));
+  else
+    hipLaunchKernelGGL(splitk_reduce_kernel<f16_t>, grid, dim3(256), 0, s, partial, plan.ksplit, n, static_cast<f16_t *>(a.y),
+                       static_cast<const f16_t *>(a.addend));
+  return launch_status();
 }
 
 }  // namespace
 
 int mfma_forward(const GemmArgs &a, hipStream_t s) { return run(a, false, s); }
 int mfma_backward(const GemmArgs &a, hipStream_t s) { return run(a, true, s); }
-size_t mfma_workspace_bytes(const GemmArgs &, bool) { return 0; }
+size_t mfma_workspace_bytes(const GemmArgs &a, bool backward)
+{
+  if (a.compute_dtype == CAIFX_F32) return 0;
+  return plan_split(a.M, backward ? a.K : a.N, backward ? a.N : a.K, a.offsets != nullptr).bytes;
+}
 
 }  // namespace caifx

@@ -99,3 +99,28 @@ def test_linearity_and_adjoint_at_full_size(orc):
     lhs = (y.double() * dy.double()).sum().item()
     rhs = (x.double() * dx.double()).sum().item()
     assert abs(lhs - rhs) <= 1e-4 * max(abs(lhs), abs(rhs))
+
+
+@pytest.mark.parametrize("M,N,K", [(40, 640, 2048),      # 5 tiles, 32 steps: 4 parts of 8 forward; dX (16 tiles, 10 steps) unsplit
+                                   (130, 1280, 1536),    # 20 tiles, 24 steps: 3 parts of 8
+                                   (100, 4096, 4096),    # 32 tiles, 64 steps: 8 parts, forward and dX
+                                   (64, 1100, 1088)])    # ragged columns; 17 steps do not divide evenly (2 parts: 9 + 8)
+@pytest.mark.parametrize("kind", ["int4", "int8pc", "int8pt"])
+def test_shared_reduction_of_few_tiles(orc, M, N, K, kind):
+    # few tiles: several workgroups share a tile's reduction through fp32 partial tiles in the caller's workspace;
+    # same operands as the plain launch, so the tight bound holds; without a workspace the plain launch runs
+    import torch
+    rng = np.random.default_rng(M + N + K)
+    _both(orc, rng, M, N, K, kind, group=64)
+    ow, dw = make_weight(orc, rng, N, K, kind, 64)
+    x = dev_as(rng.normal(0, 1, (M, K)), 2)
+    add = dev_as(rng.normal(0, 1, (M, N)), 2)
+    none = torch.empty(1, dtype=torch.uint8, device="cuda")          # too small: no sharing
+    y_split = T.qlinear_forward(x, dw, T.BF16, T.BF16, addend=add)
+    y_plain = T.qlinear_forward(x, dw, T.BF16, T.BF16, addend=add, workspace=none)
+    base = orc.round_to_dtype(orc.frozen_linear_forward(host(x), ow, 2), 2)
+    want = orc.add(base, host(add), 2)
+    # bf16 results: the fp32 sums differ in their last bits, which can move the cast's rounding by one ulp of
+    # the GEMM result (up to 2^-7 relative to it) before the Add, whose own rounding can then move by one ulp too
+    for got in (y_split, y_plain):
+        assert np.all(np.abs(host(got) - want) <= 2.0 ** -6 * np.maximum(np.maximum(np.abs(want), np.abs(base)), 1e-2))
