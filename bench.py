@@ -269,8 +269,36 @@ def compute_bound_rows(torch, T, dev, gen, capture, time_graph):
             del g
             rows["lora_base_fwd_bwd_M4096_N11008_K4096"] = {
                 "gemm_cast_add_chain_us": round(ms_c * 1e3, 1), "fused_store_us": round(ms_u * 1e3, 1)}
-    return {"prefill_gemm": rows, "fp32_compute": fp32_rows(torch, T, dev, gen, capture, time_graph),
+    return {"prefill_gemm": rows, "few_tile_gemm": few_tile_rows(torch, T, dev, gen, capture, time_graph),
+            "fp32_compute": fp32_rows(torch, T, dev, gen, capture, time_graph),
             "moe_frozen_experts": moe_rows(torch, T, dev, gen)}
+
+
+def few_tile_rows(torch, T, dev, gen, capture, time_graph):
+    """Between the decode regime and a full round of tiles (int4 g128, K = N = 4096, bf16): forward at M = 64 and
+    128 and the input gradient at M = 64, with the workspace the library asks for (workgroups share each tile's
+    reduction) and without one (plain launch)."""
+    from caif_amd import capi
+    N = K = 4096
+    w = torch.empty(N, K, device=dev).normal_(0, 0.02, generator=gen)
+    p, s = T.quantize_int4_per_group(w, 128)
+    del w
+    fw = T.FrozenWeight(p, T.W_INT4_GROUP, s, N, K, 1, 128)
+    none = torch.empty(1, dtype=torch.uint8, device=dev)
+    rows, L = {}, 16
+    for M, backward in ((64, False), (128, False), (64, True)):
+        src = torch.empty(M, N if backward else K, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16)
+        dst = torch.empty(M, K if backward else N, device=dev)
+        nb = capi.lib().caifx_qlinear_workspace_bytes(M, N, K, T.BF16, T.BF16, T.W_INT4_GROUP, int(backward))
+        ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=dev)
+        fn = T.qlinear_backward_input if backward else T.qlinear_forward
+        us = {}
+        for name, buf in (("shared_reduction_us", ws), ("plain_us", none)):
+            g = capture(lambda i, buf=buf: fn(src, fw, T.BF16, T.F32, out=dst, workspace=buf), L)
+            us[name] = round(time_graph(g, L, reps=3) * 1e3, 2)
+            del g
+        rows[f"int4_{'dx' if backward else 'fwd'}_M{M}_N{N}_K{K}"] = us
+    return rows
 
 
 def fp32_rows(torch, T, dev, gen, capture, time_graph):
