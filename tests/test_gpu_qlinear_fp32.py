@@ -55,7 +55,7 @@ def test_fp32_compute_one_hot_reads_single_weights(orc):
 
 
 def test_fp32_compute_config0_shape_and_large_m(orc):
-    # configs[0] of the baseline (K = N = 4096, fp32 X[16, 4096], int8 per-channel) and a 2048-row problem on
+    # the baseline's first configuration (K = N = 4096, fp32 X[16, 4096], int8 per-channel) and a 2048-row problem on
     # 128-row tiles, the latter on sampled rows
     rng = np.random.default_rng(21)
     N = K = 4096
