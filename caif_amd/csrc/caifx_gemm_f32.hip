@@ -6,9 +6,9 @@
 //
 // v_mfma_f32_32x32x2_f32 runs at 1/16 of the bf16 rate, so this kernel is bound by the matrix pipes long
 // before anything else and is kept simple: 256 threads, one BM x 128 tile of the result per workgroup, 32
-// deep reduction steps, one LDS buffer per operand (the next step's global loads are in flight while the
-// matrix cores work on the current one; two barriers per step cost little against the 1000-4000 MFMA
-// cycles between them).  Both operands sit in LDS reduction-major ([r][row] with the row index contiguous),
+// deep reduction steps, one LDS buffer per operand (the global loads of the next two steps are in flight in two
+// register sets while the matrix cores work on the current one; two barriers per step cost little against the
+// 1000-4000 MFMA cycles between them).  Plain and grouped (per-expert row segments) problems.  Both operands sit in LDS reduction-major ([r][row] with the row index contiguous),
 // which is what the MFMA operands read: lane (i, h) of a 32x32x2 step takes element [2p + h][i].
 // Up to 32 activation rows a workgroup takes a 32 x 32 tile with 128-deep steps and its four waves split each
 // step's reduction (partial tiles are added through LDS in a fixed order at the end): four times as many
