@@ -85,7 +85,9 @@ size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtyp
   a.x_dtype = x_dtype;
   a.compute_dtype = compute_dtype;
   a.w.kind = w_kind;
-  return mfma_workspace_bytes(a, backward != 0);
+  const size_t f32_bytes = mfma_f32_workspace_bytes(a, backward != 0);
+  const size_t bytes = mfma_workspace_bytes(a, backward != 0);
+  return f32_bytes > bytes ? f32_bytes : bytes;
 }
 
 // `addend` (optional): the matrix-core GEMM adds it in its store; every other path runs as usual and is

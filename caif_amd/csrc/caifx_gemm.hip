@@ -906,22 +906,25 @@ int run(const GemmArgs &a, bool backward, hipStream_t s)
     st = a.x_dtype == CAIFX_F32 ? pick_kind<f16_t, float>(t, int4, backward, grouped, s) : pick_kind<f16_t, f16_t>(t, int4, backward, grouped, s);
   }
   if (!split || st != CAIFX_OK) return st;
-  const int64_t n = a.M * cols;
-  const dim3 grid(static_cast<unsigned>((n + 255) / 256));
-  const float *partial = static_cast<const float *>(a.workspace);
-  if (a.y_dtype == CAIFX_F32)
-    hipLaunchKernelGGL(splitk_reduce_kernel<float>, grid, dim3(256), 0, s, partial, plan.ksplit, n, static_cast<float *>(a.y),
-                       static_cast<const float *>(a.addend));
-  else if (a.y_dtype == CAIFX_BF16)
-    hipLaunchKernelGGL(splitk_reduce_kernel<bf16_t>, grid, dim3(256), 0, s, partial, plan.ksplit, n, static_cast<bf16_t *>(a.y),
-                       static_cast<const bf16_t *>(a.addend));
-  else
-    hipLaunchKernelGGL(splitk_reduce_kernel<f16_t>, grid, dim3(256), 0, s, partial, plan.ksplit, n, static_cast<f16_t *>(a.y),
-                       static_cast<const f16_t *>(a.addend));
-  return launch_status();
+  return splitk_reduce(static_cast<const float *>(a.workspace), plan.ksplit, a.M * cols, a.y, a.y_dtype, a.addend, s);
 }
 
 }  // namespace
+
+int splitk_reduce(const float *partial, int parts, int64_t n, void *y, int y_dtype, const void *addend, hipStream_t s)
+{
+  const dim3 grid(static_cast<unsigned>((n + 255) / 256));
+  if (y_dtype == CAIFX_F32)
+    hipLaunchKernelGGL(splitk_reduce_kernel<float>, grid, dim3(256), 0, s, partial, parts, n, static_cast<float *>(y),
+                       static_cast<const float *>(addend));
+  else if (y_dtype == CAIFX_BF16)
+    hipLaunchKernelGGL(splitk_reduce_kernel<bf16_t>, grid, dim3(256), 0, s, partial, parts, n, static_cast<bf16_t *>(y),
+                       static_cast<const bf16_t *>(addend));
+  else
+    hipLaunchKernelGGL(splitk_reduce_kernel<f16_t>, grid, dim3(256), 0, s, partial, parts, n, static_cast<f16_t *>(y),
+                       static_cast<const f16_t *>(addend));
+  return launch_status();
+}
 
 int mfma_forward(const GemmArgs &a, hipStream_t s) { return run(a, false, s); }
 int mfma_backward(const GemmArgs &a, hipStream_t s) { return run(a, true, s); }

@@ -37,6 +37,10 @@ struct F32Args {
   const void *const *wq_ptrs;
   const void *const *scales_ptrs;
   int num_experts;
+  // split tile only: `parts` workgroups share a tile's reduction, part_steps 128-deep steps each (blockIdx.y is the
+  // part), and write fp32 partial tiles to d + part * M * C (d is then the caller's workspace)
+  int parts;
+  int part_steps;
 };
 
 __device__ __forceinline__ void store_result(void *p, int dt, int64_t i, float v)
@@ -80,10 +84,11 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
   const int wn = kSplit ? 0 : wave % WN;
   const int64_t R = kBackward ? g.N : g.K;
   const int64_t C = kBackward ? g.K : g.N;
-  int64_t row0 = static_cast<int64_t>(blockIdx.y) * BM;
+  int64_t row0 = kSplit ? 0 : static_cast<int64_t>(blockIdx.y) * BM;
+  const int part = kSplit ? static_cast<int>(blockIdx.y) : 0;
   int64_t row_hi = g.M;                                          // rows this workgroup may touch end here
   const int64_t col0 = static_cast<int64_t>(blockIdx.x) * kBN;
-  const int steps = static_cast<int>(R / kBK);
+  int steps = static_cast<int>(R / kBK);
   const uint8_t *wq = g.wq;
   const void *scales = g.scales;
   if (g.offsets) {
@@ -110,6 +115,15 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
   int64_t am = row0 + a_row;
   if (am >= row_hi) am = row_hi - 1;                             // rows past the end are never stored
   const XT *ap = static_cast<const XT *>(g.a) + am * R + a_col;
+  int64_t r_begin = 0;                                           // first reduction element of this workgroup's part
+  if constexpr (kSplit) {
+    if (g.parts > 1) {
+      const int first = part * g.part_steps;
+      r_begin = static_cast<int64_t>(first) * kBK;
+      steps = steps - first < g.part_steps ? steps - first : g.part_steps;
+      ap += r_begin;
+    }
+  }
   // two register sets: the loads of steps s+1 and s+2 are in flight while the matrix cores work on step s
   float areg[2][EA];
   auto load_a = [&](auto set_, int64_t r0) {
@@ -158,6 +172,7 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
     if (k + 16 > g.K) k = g.K - 16;                              // lands in LDS columns that are never stored
     flat0 = static_cast<int64_t>(b_major) * g.K + k;
   }
+  flat0 += kBackward ? r_begin * g.K : r_begin;
   const int64_t flat_step = kBackward ? static_cast<int64_t>(kBK) * g.K : kBK;
   const float *s32 = static_cast<const float *>(scales);
   const f16_t *s16 = static_cast<const f16_t *>(scales);
@@ -298,7 +313,7 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
       for (int w = 1; w < 4; ++w) v += As[(w * 16 + r) * 64 + ln];
       const int64_t row = row0 + 8 * (r >> 2) + 4 * (ln >> 5) + (r & 3);
       const int64_t col = col0 + (ln & 31);
-      if (row < row_hi && col < C) store_result(g.d, g.d_dtype, row * C + col, v);
+      if (row < row_hi && col < C) store_result(g.d, g.d_dtype, static_cast<int64_t>(part) * g.M * C + row * C + col, v);
     }
     return;
   }
@@ -334,8 +349,8 @@ int launch_bm(const F32Args &f, hipStream_t s)
   }
   // up to 32 rows: 32-column tiles whose waves split the reduction (128-deep steps)
   if (f.M <= 32 && R % 128 == 0) {
-    hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 32, 128>), dim3(static_cast<unsigned>((C + 31) / 32), 1), dim3(256), 0,
-                       s, f);
+    hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 32, 128>),
+                       dim3(static_cast<unsigned>((C + 31) / 32), static_cast<unsigned>(f.parts)), dim3(256), 0, s, f);
     return launch_status();
   }
   // 128-row tiles once there are enough of them to give every compute unit one; below that 32-row tiles
@@ -359,6 +374,33 @@ int launch_kind(const F32Args &f, bool int4, bool backward, hipStream_t s)
   if (int4) return backward ? launch_bm<XT, true, false, true>(f, s) : launch_bm<XT, true, false, false>(f, s);
   if (f.period > 1) return backward ? launch_bm<XT, false, true, true>(f, s) : launch_bm<XT, false, true, false>(f, s);
   return backward ? launch_bm<XT, false, false, true>(f, s) : launch_bm<XT, false, false, false>(f, s);
+}
+
+// Up to 32 rows there are C / 32 split tiles, 128 at C = 4096: a chain of R / 128 dependent steps on half of the
+// chip.  With a workspace from the caller up to 4 workgroups share a tile's reduction (at least 8 steps each, about
+// one workgroup per compute unit in total) and a second launch adds their partial tiles in a fixed order.
+struct F32Plan {
+  int parts;
+  int part_steps;
+  size_t bytes;
+};
+F32Plan plan_f32(int64_t M, int64_t C, int64_t R, bool grouped)
+{
+  F32Plan p{1, 0, 0};
+  if (grouped || M > 32 || R % 128 != 0) return p;
+  const int64_t tiles = (C + 31) / 32;
+  const int64_t steps = R / 128;
+  int64_t k = 256 / tiles;
+  if (k > 4) k = 4;
+  if (k > steps / 8) k = steps / 8;
+  if (k < 2) return p;
+  const int64_t per = (steps + k - 1) / k;
+  k = (steps + per - 1) / per;
+  if (k < 2) return p;
+  p.parts = static_cast<int>(k);
+  p.part_steps = static_cast<int>(per);
+  p.bytes = static_cast<size_t>(k) * static_cast<size_t>(M) * static_cast<size_t>(C) * sizeof(float);
+  return p;
 }
 
 int run_f32(const GemmArgs &a, bool backward, hipStream_t s)
@@ -407,13 +449,32 @@ int run_f32(const GemmArgs &a, bool backward, hipStream_t s)
   } else {
     return CAIFX_ERR_UNSUPPORTED;
   }
-  if (a.x_dtype == CAIFX_F32) return launch_kind<float>(f, int4, backward, s);
-  if (a.x_dtype == CAIFX_BF16) return launch_kind<bf16_t>(f, int4, backward, s);
-  if (a.x_dtype == CAIFX_F16) return launch_kind<f16_t>(f, int4, backward, s);
-  return CAIFX_ERR_UNSUPPORTED;
+  f.parts = 1;
+  const int64_t cols = backward ? a.K : a.N;
+  const F32Plan plan = plan_f32(a.M, cols, R, grouped);
+  const bool shared = plan.parts > 1 && a.workspace && a.workspace_bytes >= plan.bytes && aligned_to(a.workspace, 4);
+  if (shared) {
+    f.parts = plan.parts;
+    f.part_steps = plan.part_steps;
+    f.d = a.workspace;
+    f.d_dtype = CAIFX_F32;
+  }
+  int st;
+  if (a.x_dtype == CAIFX_F32) st = launch_kind<float>(f, int4, backward, s);
+  else if (a.x_dtype == CAIFX_BF16) st = launch_kind<bf16_t>(f, int4, backward, s);
+  else if (a.x_dtype == CAIFX_F16) st = launch_kind<f16_t>(f, int4, backward, s);
+  else return CAIFX_ERR_UNSUPPORTED;
+  if (!shared || st != CAIFX_OK) return st;
+  return splitk_reduce(static_cast<const float *>(a.workspace), plan.parts, a.M * cols, a.y, a.y_dtype, nullptr, s);
 }
 
 }  // namespace
+
+size_t mfma_f32_workspace_bytes(const GemmArgs &a, bool backward)
+{
+  if (a.compute_dtype != CAIFX_F32) return 0;
+  return plan_f32(a.M, backward ? a.K : a.N, backward ? a.N : a.K, a.offsets != nullptr).bytes;
+}
 
 int mfma_f32_forward(const GemmArgs &a, hipStream_t s) { return run_f32(a, false, s); }
 int mfma_f32_backward(const GemmArgs &a, hipStream_t s) { return run_f32(a, true, s); }

@@ -60,5 +60,10 @@ size_t mfma_workspace_bytes(const GemmArgs &a, bool backward);
 // int4 groups below 16 or not a power of two, int8 scale vectors shorter than 32 or not a multiple of 4 long.
 int mfma_f32_forward(const GemmArgs &a, hipStream_t s);
 int mfma_f32_backward(const GemmArgs &a, hipStream_t s);
+size_t mfma_f32_workspace_bytes(const GemmArgs &a, bool backward);
+
+// y[i] = T(partial[0][i] + partial[1][i] + ...) in that order for i < n, T = y_dtype, then the optional addend
+// with the roundings of a cast and an Add: the second launch of a reduction shared among workgroups.
+int splitk_reduce(const float *partial, int parts, int64_t n, void *y, int y_dtype, const void *addend, hipStream_t s);
 
 }  // namespace caifx
