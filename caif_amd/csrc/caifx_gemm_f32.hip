@@ -21,6 +21,7 @@ namespace caifx {
 namespace {
 
 constexpr int kStep = 32;    // the reduction advances in multiples of this (host-side checks, scale-index steps)
+constexpr int kSplitTileRows = 128;   // up to this many rows the 32 x 32 split tile is used (M = 64: 256 workgroups instead of 64)
 
 struct F32Args {
   int64_t M, N, K;
@@ -37,7 +38,7 @@ struct F32Args {
   const void *const *wq_ptrs;
   const void *const *scales_ptrs;
   int num_experts;
-  // split tile only: `parts` workgroups share a tile's reduction, part_steps 128-deep steps each (blockIdx.y is the
+  // split tile only: `parts` workgroups share a tile's reduction, part_steps 128-deep steps each (blockIdx.z is the
   // part), and write fp32 partial tiles to d + part * M * C (d is then the caller's workspace)
   int parts;
   int part_steps;
@@ -84,8 +85,8 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
   const int wn = kSplit ? 0 : wave % WN;
   const int64_t R = kBackward ? g.N : g.K;
   const int64_t C = kBackward ? g.K : g.N;
-  int64_t row0 = kSplit ? 0 : static_cast<int64_t>(blockIdx.y) * BM;
-  const int part = kSplit ? static_cast<int>(blockIdx.y) : 0;
+  int64_t row0 = static_cast<int64_t>(blockIdx.y) * BM;
+  const int part = kSplit ? static_cast<int>(blockIdx.z) : 0;
   int64_t row_hi = g.M;                                          // rows this workgroup may touch end here
   const int64_t col0 = static_cast<int64_t>(blockIdx.x) * kBN;
   int steps = static_cast<int>(R / kBK);
@@ -347,10 +348,11 @@ int launch_bm(const F32Args &f, hipStream_t s)
     else hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 128, 32>), grid, dim3(256), 0, s, f);
     return launch_status();
   }
-  // up to 32 rows: 32-column tiles whose waves split the reduction (128-deep steps)
-  if (f.M <= 32 && R % 128 == 0) {
+  // few rows: 32 x 32 tiles whose waves split the reduction (128-deep steps)
+  if (f.M <= kSplitTileRows && R % 128 == 0) {
     hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 32, 128>),
-                       dim3(static_cast<unsigned>((C + 31) / 32), static_cast<unsigned>(f.parts)), dim3(256), 0, s, f);
+                       dim3(static_cast<unsigned>((C + 31) / 32), static_cast<unsigned>((f.M + 31) / 32), static_cast<unsigned>(f.parts)),
+                       dim3(256), 0, s, f);
     return launch_status();
   }
   // 128-row tiles once there are enough of them to give every compute unit one; below that 32-row tiles
@@ -376,7 +378,7 @@ int launch_kind(const F32Args &f, bool int4, bool backward, hipStream_t s)
   return backward ? launch_bm<XT, false, false, true>(f, s) : launch_bm<XT, false, false, false>(f, s);
 }
 
-// Up to 32 rows there are C / 32 split tiles, 128 at C = 4096: a chain of R / 128 dependent steps on half of the
+// Up to 32 rows there are C / 32 split tiles, 128 at C = 4096 (more rows: that many per 32 rows): a chain of R / 128 dependent steps on half of the
 // chip.  With a workspace from the caller up to 4 workgroups share a tile's reduction (at least 8 steps each, about
 // one workgroup per compute unit in total) and a second launch adds their partial tiles in a fixed order.
 struct F32Plan {
@@ -387,8 +389,9 @@ struct F32Plan {
 F32Plan plan_f32(int64_t M, int64_t C, int64_t R, bool grouped)
 {
   F32Plan p{1, 0, 0};
-  if (grouped || M > 32 || R % 128 != 0) return p;
-  const int64_t tiles = (C + 31) / 32;
+  if (grouped || M > kSplitTileRows || R % 128 != 0) return p;
+  const int64_t tiles = ((C + 31) / 32) * ((M + 31) / 32);
+  if (tiles > 128) return p;
   const int64_t steps = R / 128;
   int64_t k = 256 / tiles;
   if (k > 4) k = 4;
