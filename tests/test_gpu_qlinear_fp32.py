@@ -18,7 +18,9 @@ TOL = 1e-4
 @pytest.mark.parametrize("M,N,K", [(5, 192, 256),       # 32-row tiles, one partial row tile
                                    (70, 160, 96),       # N and K below a column tile; K % 128 != 0 (input gradient)
                                    (300, 416, 512),     # several row tiles, N % 128 != 0
-                                   (33, 100, 64)])      # N % 32 != 0: the input gradient takes the shape-agnostic kernel
+                                   (33, 100, 64),       # N % 32 != 0: the input gradient takes the shape-agnostic kernel
+                                   (100, 256, 512),     # 32 x 32 split tiles, four row tiles (the last one partial)
+                                   (70, 384, 2048)])    # ... with two workgroups sharing each tile's reduction (forward)
 def test_fp32_compute_forward_and_input_gradient(orc, kind, group, M, N, K):
     rng = np.random.default_rng(M * 1000 + N + K + group)
     if kind == "int4" and (N * K) % group:
