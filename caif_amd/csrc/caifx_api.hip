@@ -1,9 +1,32 @@
 // extern "C" entry points of the dequant-GEMM seam: argument validation and kernel choice.
 #include "caifx_internal.hpp"
 
+#include <atomic>
+
 using namespace caifx;
 
+// Scratch of caifx_qlinear_forward_static: part of the device image, so every GPU the library is loaded on has
+// its own copy at its own address.  In host code `static_scratch` is only a handle for hipGetSymbolAddress, not a
+// device address; the address is looked up once per device and only that address is ever handed to a launch.
+static __device__ __align__(256) unsigned char static_scratch[CAIFX_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<void *> static_scratch_ptr[kMaxDevices];
+
+// Address of the current device's copy (nullptr on failure).  Two threads racing on a device's first call both
+// look the same address up and store the same value.
+void *static_scratch_on_current_device()
+{
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void *p = static_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch)) != hipSuccess || !p) return nullptr;
+  static_scratch_ptr[dev].store(p, std::memory_order_release);
+  return p;
+}
 
 int validate_weight(int64_t N, int64_t K, int w_kind, const void *scales, int64_t scale_period, int group_size)
 {
@@ -69,6 +92,7 @@ const char *caifx_status_string(int status)
     case CAIFX_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
     case CAIFX_ERR_LAUNCH_FAILED: return "kernel launch failed";
     case CAIFX_ERR_MISALIGNED: return "misaligned pointer";
+    case CAIFX_ERR_SCRATCH_EXCEEDED: return "problem needs more scratch than the library's static buffer holds";
     default: return "unknown status";
   }
 }
@@ -157,6 +181,23 @@ int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K, const void *x, int x_
 {
   return forward_impl(M, N, K, x, x_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, y, y_dtype,
                       nullptr, workspace, workspace_bytes, stream);
+}
+
+int caifx_qlinear_forward_static(int64_t M, int64_t N, int64_t K, const void *x, int x_dtype, int compute_dtype,
+                                 const void *wq, int w_kind, const void *scales, int64_t scale_period, int group_size,
+                                 void *y, int y_dtype, caifx_stream_t stream)
+{
+  const size_t need = (M > 0 && N > 0 && K > 0 && valid_dtype(x_dtype) && valid_dtype(compute_dtype))
+                          ? caifx_qlinear_workspace_bytes(M, N, K, x_dtype, compute_dtype, w_kind, 0)
+                          : 0;
+  if (need > CAIFX_STATIC_SCRATCH_BYTES) return CAIFX_ERR_SCRATCH_EXCEEDED;
+  void *ws = nullptr;
+  if (need > 0) {
+    ws = static_scratch_on_current_device();
+    if (!ws) return CAIFX_ERR_LAUNCH_FAILED;
+  }
+  return forward_impl(M, N, K, x, x_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, y, y_dtype,
+                      nullptr, ws, need, stream);
 }
 
 int caifx_qlinear_forward_add(int64_t M, int64_t N, int64_t K, const void *x, int x_dtype, int compute_dtype,

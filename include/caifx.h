@@ -48,7 +48,8 @@ enum caifx_status {
   CAIFX_ERR_UNSUPPORTED = 2,             /* a combination this build has no kernel for */
   CAIFX_ERR_WORKSPACE_TOO_SMALL = 3,
   CAIFX_ERR_LAUNCH_FAILED = 4,           /* hipGetLastError() != hipSuccess after a launch */
-  CAIFX_ERR_MISALIGNED = 5               /* pointer not aligned to its element type */
+  CAIFX_ERR_MISALIGNED = 5,              /* pointer not aligned to its element type */
+  CAIFX_ERR_SCRATCH_EXCEEDED = 6         /* the problem needs more scratch than the library's static buffer holds */
 };
 
 /* Float element types (CAIF_DataType::Float32 / Float16 / BFloat16). */
@@ -173,6 +174,24 @@ CAIFX_API int caifx_qlinear_backward_input_add(int64_t M, int64_t N, int64_t K,
  * workspace the calls run without that sharing, only slower. */
 CAIFX_API size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtype, int compute_dtype,
                                      int w_kind, int backward);
+
+/* caifx_qlinear_forward for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc) and so have no workspace to pass: the fp32 partial tiles of a
+ * shared reduction go to a buffer of CAIFX_STATIC_SCRATCH_BYTES that is part of the library's device image (one
+ * copy per GPU, held until the process ends) instead of the caller's workspace.  It has no counterpart in the
+ * reference, whose layers allocate freely.  Same arguments, kernels and results (bit for bit) as
+ * caifx_qlinear_forward called with a workspace of caifx_qlinear_workspace_bytes(..., backward = 0) bytes.
+ * A problem for which that size exceeds CAIFX_STATIC_SCRATCH_BYTES returns CAIFX_ERR_SCRATCH_EXCEEDED and
+ * launches nothing (use caifx_qlinear_forward then; with a null workspace it runs without sharing).
+ * The call itself allocates and frees nothing.  Every call on one GPU uses that GPU's one buffer: calls on
+ * different streams of the same GPU that may overlap race on it; calls on one stream are ordered and need no
+ * clearing in between (every partial tile is written in full before it is read). */
+#define CAIFX_STATIC_SCRATCH_BYTES (8u << 20)
+CAIFX_API int caifx_qlinear_forward_static(int64_t M, int64_t N, int64_t K,
+                                 const void *x, int x_dtype, int compute_dtype,
+                                 const void *wq, int w_kind, const void *scales, int64_t scale_period,
+                                 int group_size,
+                                 void *y, int y_dtype, caifx_stream_t stream);
 
 /* The per-expert loop of CAIF_DeviceMoELayer over frozen experts
  * (src/caif_device_moe_layer.cpp:534-557 forward, :754-778 backward) as ONE
