@@ -269,6 +269,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
   constexpr int kPlanes = 3;              // 2 would give 14-bit activations; the third plane costs 4 of 12 MFMAs per block
   i32x4_t dg[kInt4 ? 1 : kSteps][kPlanes];
   float ur[4] = {1.0f, 1.0f, 1.0f, 1.0f};     // unit of the activation rows 4q..4q+3 this lane holds results of
+  bool poison[4] = {false, false, false, false};   // those rows have a non-finite scaled activation in this wave's k range
   if constexpr (!kInt4) {
     __syncthreads();       // svec is complete
     // four consecutive x' values: quad c (0..3) of step t
@@ -283,6 +284,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
       for (int i = 0; i < 4; ++i) v[i] *= sc4[i];
     };
     float mx = 0.0f;
+    bool finite = true;
 #pragma unroll
     for (int t = 0; t < kSteps; ++t)
 #pragma unroll
@@ -290,10 +292,19 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
         float v[4];
         xprime4(t, c, v);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fabsf(v[i]));
+        for (int i = 0; i < 4; ++i) {
+          mx = fmaxf(mx, fabsf(v[i]));                       // ignores a NaN
+          finite = finite && fabsf(v[i]) <= 3.4028235e38f;    // false for NaN and infinities
+        }
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16));
     mx = fmaxf(mx, __shfl_xor(mx, 32));      // over the four k quarters: row j's largest |x'| in this wave's k range
+    // A NaN or an infinity among row j's scaled activations has no digits.  The reference's GEMM returns NaN or an
+    // infinity in every output of that activation row; here this wave's share of them, and so their sum, is NaN.
+    const int bad = (__ballot(!finite) >> j & 0x0001000100010001ull) != 0 ? 1 : 0;
+    mx = bad ? 1.0f : mx;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) poison[r] = __shfl(bad, 4 * q + r) != 0;
     int e = 0;
     (void)frexpf(mx, &e);                     // mx = f * 2^e, f in [0.5, 1)
     const float unit = mx > 0.0f ? ldexpf(1.0f, e - 6) : 1.0f;    // |x'| / unit <= 64
@@ -378,7 +389,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
               float v = static_cast<float>(s0[r]);
               v = __builtin_fmaf(static_cast<float>(s1[r]), 1.0f / 128.0f, v);
               if constexpr (kPlanes == 3) v = __builtin_fmaf(static_cast<float>(s2[r]), 1.0f / 16384.0f, v);
-              tot[u][r] = v * ur[r];
+              tot[u][r] = poison[r] ? __builtin_nanf("") : v * ur[r];
             }
           }
         }

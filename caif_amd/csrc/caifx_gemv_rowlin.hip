@@ -70,6 +70,7 @@ struct RowArgs {
   int cpr;              // chunks (one load instruction of a wave) per weight row
   int xpitch;           // staged activations: elements per row (cpr * k-per-chunk)
   int digits;           // int8, one activation row: take the integer-matrix-core kernel
+  int round_x;          // that kernel only: activations pass through this dtype first (caifx_dtype), -1 = they are of it already
 };
 
 template <typename CT, typename XT>
@@ -677,6 +678,14 @@ __global__ __launch_bounds__(kDigitWaves * 64) void rowlin_int8_digits_kernel(Ro
     const XT *xg = static_cast<const XT *>(a.x) + (wave * 64 + lane) * 16;
 #pragma unroll
     for (int t = 0; t < 16; ++t) xv[t] = to_f32<XT>(xg[t]);
+    // the layer casts its input to the compute dtype before the GEMM (src/caif_device_frozen_linear.cpp:459)
+    if (a.round_x == CAIFX_BF16) {
+#pragma unroll
+      for (int t = 0; t < 16; ++t) xv[t] = round_through<bf16_t>(xv[t]);
+    } else if (a.round_x == CAIFX_F16) {
+#pragma unroll
+      for (int t = 0; t < 16; ++t) xv[t] = round_through<f16_t>(xv[t]);
+    }
     if constexpr (kVec) {
       const float *sp = static_cast<const float *>(a.scales);
       // 32-bit arithmetic: cls < N / 256 and K <= 4096, so cls * K + k stays far below 2^31
@@ -716,8 +725,13 @@ __global__ __launch_bounds__(kDigitWaves * 64) void rowlin_int8_digits_kernel(Ro
         for (int t = 0; t < 4; ++t) xv[4 * q + t] *= scv[q][t];
     }
     float m = 0.0f;
+    bool finite = true;
 #pragma unroll
-    for (int t = 0; t < 16; ++t) m = fmaxf(m, fabsf(xv[t]));
+    for (int t = 0; t < 16; ++t) {
+      m = fmaxf(m, fabsf(xv[t]));                       // ignores a NaN
+      finite = finite && fabsf(xv[t]) <= 3.4028235e38f;  // false for NaN and infinities
+    }
+    m = finite ? m : __builtin_inff();
     m = fmaxf(m, __shfl_xor(m, 16));
     m = fmaxf(m, __shfl_xor(m, 32));
     if (lane < 16) mx[wave][lane] = m;
@@ -726,13 +740,17 @@ __global__ __launch_bounds__(kDigitWaves * 64) void rowlin_int8_digits_kernel(Ro
 
   // power-of-two unit of diagonal element i: the largest |x'| of its CPR*64 values maps into [32, 64]
   float unit;
+  bool poisoned;       // wave uniform, and the same in every wave of the workgroup
   {
     float m = 0.0f;
 #pragma unroll
     for (int c = 0; c < CPR; ++c) m = fmaxf(m, mx[c][lane & 15]);
+    // A NaN or an infinity among the scaled activations has no digits.  The reference's GEMM returns NaN or an
+    // infinity in every output then (each output multiplies every activation); here every output becomes NaN.
+    poisoned = __any(!(m <= 3.4028235e38f));
     int e = 0;
-    (void)frexpf(m, &e);                      // m = f * 2^e, f in [0.5, 1)
-    unit = m > 0.0f ? ldexpf(1.0f, e - 6) : 1.0f;
+    (void)frexpf(poisoned ? 1.0f : m, &e);    // m = f * 2^e, f in [0.5, 1)
+    unit = (m > 0.0f && !poisoned) ? ldexpf(1.0f, e - 6) : 1.0f;
   }
   if (has_chunk) {
     // n = round(x' / unit * 2^14) as the low mantissa bits of x' * (2^14 / unit) + 1.5 * 2^23 (|n| <= 2^20);
@@ -795,7 +813,7 @@ __global__ __launch_bounds__(kDigitWaves * 64) void rowlin_int8_digits_kernel(Ro
       issue(d, r + D);
     }
   }
-  if (lane < nrows) static_cast<float *>(a.y)[cls + V * (i0 + lane)] = res;
+  if (lane < nrows) static_cast<float *>(a.y)[cls + V * (i0 + lane)] = poisoned ? __builtin_nanf("") : res;
 }
 
 
@@ -1100,6 +1118,7 @@ int rowlin_forward(const GemmArgs &g, hipStream_t s)
     ra.waves_per_class = static_cast<int>((rows_class + ra.rows_per_wave - 1) / ra.rows_per_wave);
     if (digits) {
       ra.digits = 1;
+      ra.round_x = g.x_dtype != g.compute_dtype ? g.compute_dtype : -1;
       ra.waves_per_class = (ra.waves_per_class + kDigitWaves - 1) / kDigitWaves * kDigitWaves;      // a workgroup stays inside one class
     }
     ra.total_waves = ra.waves_per_class * ra.row_stride;

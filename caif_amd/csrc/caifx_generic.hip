@@ -65,23 +65,25 @@ __global__ void generic_forward_kernel(GemmArgs a)
     wq = a.wq_ptrs[e];
     scales = a.scales_ptrs ? a.scales_ptrs[e] : nullptr;
   }
-  const int64_t m0 = row_lo + static_cast<int64_t>(blockIdx.y) * kMB;
-  if (n >= a.N || m0 >= row_hi) return;
-  const int mcnt = static_cast<int>(row_hi - m0 < kMB ? row_hi - m0 : kMB);
-  float acc[kMB];
+  if (n >= a.N) return;
+  // blocks of kMB rows are strided over gridDim.y, which the launch caps at the grid limit
+  for (int64_t m0 = row_lo + static_cast<int64_t>(blockIdx.y) * kMB; m0 < row_hi; m0 += static_cast<int64_t>(gridDim.y) * kMB) {
+    const int mcnt = static_cast<int>(row_hi - m0 < kMB ? row_hi - m0 : kMB);
+    float acc[kMB];
 #pragma unroll
-  for (int i = 0; i < kMB; ++i) acc[i] = 0.0f;
-  for (int64_t k = lane; k < a.K; k += 64) {
-    const float wv = weight_rt(a.w, wq, scales, n * a.K + k, a.compute_dtype);
+    for (int i = 0; i < kMB; ++i) acc[i] = 0.0f;
+    for (int64_t k = lane; k < a.K; k += 64) {
+      const float wv = weight_rt(a.w, wq, scales, n * a.K + k, a.compute_dtype);
 #pragma unroll
-    for (int i = 0; i < kMB; ++i)
-      if (i < mcnt) acc[i] = __builtin_fmaf(round_rt(load_rt(a.x, a.x_dtype, (m0 + i) * a.K + k), a.compute_dtype), wv, acc[i]);
-  }
+      for (int i = 0; i < kMB; ++i)
+        if (i < mcnt) acc[i] = __builtin_fmaf(round_rt(load_rt(a.x, a.x_dtype, (m0 + i) * a.K + k), a.compute_dtype), wv, acc[i]);
+    }
 #pragma unroll
-  for (int i = 0; i < kMB; ++i) {
-    float v = acc[i];
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    if (lane == 0 && i < mcnt) store_rt(a.y, a.y_dtype, (m0 + i) * a.N + n, v);
+    for (int i = 0; i < kMB; ++i) {
+      float v = acc[i];
+      for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+      if (lane == 0 && i < mcnt) store_rt(a.y, a.y_dtype, (m0 + i) * a.N + n, v);
+    }
   }
 }
 
@@ -103,40 +105,49 @@ __global__ void generic_backward_kernel(GemmArgs a)
     wq = a.wq_ptrs[e];
     scales = a.scales_ptrs ? a.scales_ptrs[e] : nullptr;
   }
-  const int64_t m0 = row_lo + static_cast<int64_t>(blockIdx.y) * kMB;
-  if (k >= a.K || m0 >= row_hi) return;
-  const int mcnt = static_cast<int>(row_hi - m0 < kMB ? row_hi - m0 : kMB);
-  float acc[kMB];
+  if (k >= a.K) return;
+  for (int64_t m0 = row_lo + static_cast<int64_t>(blockIdx.y) * kMB; m0 < row_hi; m0 += static_cast<int64_t>(gridDim.y) * kMB) {
+    const int mcnt = static_cast<int>(row_hi - m0 < kMB ? row_hi - m0 : kMB);
+    float acc[kMB];
 #pragma unroll
-  for (int i = 0; i < kMB; ++i) acc[i] = 0.0f;
-  for (int64_t n = 0; n < a.N; ++n) {
-    const float wv = weight_rt(a.w, wq, scales, n * a.K + k, a.compute_dtype);
+    for (int i = 0; i < kMB; ++i) acc[i] = 0.0f;
+    for (int64_t n = 0; n < a.N; ++n) {
+      const float wv = weight_rt(a.w, wq, scales, n * a.K + k, a.compute_dtype);
+#pragma unroll
+      for (int i = 0; i < kMB; ++i)
+        if (i < mcnt) acc[i] = __builtin_fmaf(round_rt(load_rt(a.x, a.x_dtype, (m0 + i) * a.N + n), a.compute_dtype), wv, acc[i]);
+    }
 #pragma unroll
     for (int i = 0; i < kMB; ++i)
-      if (i < mcnt) acc[i] = __builtin_fmaf(round_rt(load_rt(a.x, a.x_dtype, (m0 + i) * a.N + n), a.compute_dtype), wv, acc[i]);
+      if (i < mcnt) store_rt(a.y, a.y_dtype, (m0 + i) * a.K + k, acc[i]);
   }
-#pragma unroll
-  for (int i = 0; i < kMB; ++i)
-    if (i < mcnt) store_rt(a.y, a.y_dtype, (m0 + i) * a.K + k, acc[i]);
 }
 
 }  // namespace
 
 // a.M is the row count for the plain call, or an upper bound of any one expert's segment
 // length for the grouped call (offsets != nullptr, num_experts > 0).
+// Grid limits: y and z hold at most 65535 blocks.  Row blocks beyond that are reached by the kernels' stride over
+// gridDim.y; more experts than that have no launch here.
+unsigned generic_row_blocks(int64_t M)
+{
+  const int64_t blocks = (M + kMB - 1) / kMB;
+  return static_cast<unsigned>(blocks < 1 ? 1 : (blocks > 65535 ? 65535 : blocks));
+}
+
 int generic_forward(const GemmArgs &a, hipStream_t s)
 {
   const int waves = 4;
-  dim3 grid(static_cast<unsigned>((a.N + waves - 1) / waves), static_cast<unsigned>((a.M + kMB - 1) / kMB),
-            a.offsets ? a.num_experts : 1);
+  if (a.offsets && a.num_experts > 65535) return CAIFX_ERR_UNSUPPORTED;
+  dim3 grid(static_cast<unsigned>((a.N + waves - 1) / waves), generic_row_blocks(a.M), a.offsets ? a.num_experts : 1);
   hipLaunchKernelGGL(generic_forward_kernel, grid, dim3(waves * 64), 0, s, a);
   return launch_status();
 }
 
 int generic_backward(const GemmArgs &a, hipStream_t s)
 {
-  dim3 grid(static_cast<unsigned>((a.K + 255) / 256), static_cast<unsigned>((a.M + kMB - 1) / kMB),
-            a.offsets ? a.num_experts : 1);
+  if (a.offsets && a.num_experts > 65535) return CAIFX_ERR_UNSUPPORTED;
+  dim3 grid(static_cast<unsigned>((a.K + 255) / 256), generic_row_blocks(a.M), a.offsets ? a.num_experts : 1);
   hipLaunchKernelGGL(generic_backward_kernel, grid, dim3(256), 0, s, a);
   return launch_status();
 }

@@ -215,20 +215,16 @@ class CAIF_DeviceMoEFrozenExpertBank
         _input_dim=experts[0]->Config().InputDim();
         _hidden_dim=experts[0]->Config().HiddenDim();
         _num_experts=static_cast<int>(experts.size());
-        std::vector<const void*> ptrs;
         for(int which=0;which<3;++which)
         {
-          std::vector<const void*> w,s;
           for(Expert_t *e:experts)
           {
             if(e->Config().UseGated()==false){THROW_CAIFE("MoEFrozenExpertBank: experts must be gated");}
             const auto &sub=e->SubLayers();
-            const CAIF_DeviceFrozenLinearBase *b=which==0?sub.gate.get():(which==1?sub.up.get():sub.down.get());
-            Describe(b,which,w,s);
+            _subs[which].push_back(which==0?sub.gate.get():(which==1?sub.up.get():sub.down.get()));
           }
-          Upload(w,_wq_ptrs[which]);
-          Upload(s,_scale_ptrs[which]);
         }
+        Refresh();
       }
       CAIF_CATCH_BLOCK()
     }
@@ -239,6 +235,7 @@ class CAIF_DeviceMoEFrozenExpertBank
     {
       try
       {
+        Refresh();
         const uint32_t rows=x.Shape()[0];
         const Dtype_e sd=CAIF_DtypeOf<StorageT>::value;
         CAIF_DeviceTensor up_out=CAIF_DeviceTensor::Zeros({rows,_hidden_dim},*_stream,sd);
@@ -266,6 +263,7 @@ class CAIF_DeviceMoEFrozenExpertBank
       try
       {
         if(_gate_out.IsEmpty()==true){THROW_CAIFE("MoEFrozenExpertBank::Backward: must call Forward(training=true) first");}
+        Refresh();
         const uint32_t rows=grad_out.Shape()[0];
         const Dtype_e sd=CAIF_DtypeOf<StorageT>::value;
         const std::vector<uint32_t> hs={rows,_hidden_dim};
@@ -294,6 +292,33 @@ class CAIF_DeviceMoEFrozenExpertBank
   private:
     struct Kind_t{int kind=-1;int64_t period=1;int group=0;uint32_t in=0;uint32_t out=0;};
 
+    // The grouped launches read the experts' weights through device arrays of device addresses.  A sub-layer
+    // under the HostPinned offload policy frees its device copy in Evict() and gets a new one, at a new address,
+    // in Prefetch() (src/caif_device_frozen_linear.cpp:145-232), so the addresses are gathered again before every
+    // pass and uploaded when any of them has moved; an expert that is not resident throws like the layer's own
+    // Forward does (:391-396).
+    void Refresh()
+    {
+      for(int which=0;which<3;++which)
+      {
+        std::vector<const void*> w,s;
+        for(const CAIF_DeviceFrozenLinearBase *b:_subs[which])
+        {
+          Describe(b,which,w,s);
+        }
+        if(w!=_host_wq[which])
+        {
+          Upload(w,_wq_ptrs[which]);
+          _host_wq[which]=w;
+        }
+        if(s!=_host_scales[which])
+        {
+          Upload(s,_scale_ptrs[which]);
+          _host_scales[which]=s;
+        }
+      }
+    }
+
     void Describe(const CAIF_DeviceFrozenLinearBase *b,int which,std::vector<const void*> &w,std::vector<const void*> &s)
     {
       const void *wq=nullptr;
@@ -314,6 +339,11 @@ class CAIF_DeviceMoEFrozenExpertBank
       else
       {
         THROW_CAIFE("MoEFrozenExpertBank: sub-layer must be an int8 or int4 frozen linear of the bank's ComputeT");
+      }
+      if(b->OffloadPolicy()==CAIF_OffloadPolicy::CAIF_OffloadPolicy_e::HostPinned_e&&b->IsPrefetched()==false)
+      {
+        THROW_CAIFE("MoEFrozenExpertBank: an expert's weight is not on the device (HostPinned policy)."
+                    " The block-level scheduler must call Prefetch(stream) before the bank runs.");
       }
       if(wq==nullptr){THROW_CAIFE("MoEFrozenExpertBank: sub-layer weight not loaded");}
       if(w.empty()==true)
@@ -380,6 +410,9 @@ class CAIF_DeviceMoEFrozenExpertBank
     uint32_t _hidden_dim=0;
     int _num_experts=0;
     Kind_t _kinds[3];
+    std::vector<const CAIF_DeviceFrozenLinearBase*> _subs[3];      // borrowed: gate, up, down of every expert
+    std::vector<const void*> _host_wq[3];                          // what _wq_ptrs / _scale_ptrs hold right now
+    std::vector<const void*> _host_scales[3];
     CAIF_DeviceTensor _wq_ptrs[3];
     CAIF_DeviceTensor _scale_ptrs[3];
     CAIF_DeviceTensor _gate_out;

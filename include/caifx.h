@@ -126,7 +126,9 @@ CAIFX_API int caifx_dequantize_int4(const void *packed_data, const void *scales,
  * compute_dtype is the layer's ComputeT.  No dense copy of W is ever written.
  * With up to 32 rows and a 16-bit compute type the memory-bound kernels skip the rounding of code * scale
  * to the compute type for int8 and for int4 with groups of 128 or more (the products with x are formed
- * exactly instead): results then differ from the formula above by that rounding, about 2e-3 of max|y|. */
+ * exactly instead): results then differ from the formula above by that rounding, about 2e-3 of max|y|.
+ * In the int8 kernels of that class a NaN or an infinity among the activations of a row turns every result of
+ * that row into NaN (the formula above gives NaN or an infinity in each of them). */
 CAIFX_API int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K,
                           const void *x, int x_dtype, int compute_dtype,
                           const void *wq, int w_kind, const void *scales, int64_t scale_period,
@@ -170,8 +172,9 @@ CAIFX_API int caifx_qlinear_backward_input_add(int64_t M, int64_t N, int64_t K,
  * backward != 0 asks for caifx_qlinear_backward_input.  Nonzero for 16-bit compute types when the result has
  * fewer 128 x 128 tiles than the chip has compute units: up to 8 workgroups then share a tile's reduction through
  * fp32 partial tiles in the workspace (16-byte aligned) and a second launch adds them in a fixed order (results do
- * not depend on scheduling).  The fp32 compute type does the same for up to 32 rows.  With a smaller or null
- * workspace the calls run without that sharing, only slower. */
+ * not depend on scheduling).  The fp32 compute type does the same for up to 128 rows.  With a smaller or null
+ * workspace the calls run without that sharing, only slower, and the sums are formed in a different order, so
+ * the last bits of a result may differ between a call with and a call without the workspace. */
 CAIFX_API size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtype, int compute_dtype,
                                      int w_kind, int backward);
 

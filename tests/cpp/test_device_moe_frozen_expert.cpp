@@ -94,6 +94,24 @@ static void GpuTests()
     }
     Report("bank forward equals the per-expert loop",RelToMax(yb,yl)<=1e-2f);
     Report("bank backward equals the per-expert loop",RelToMax(db,dl)<=1e-2f);
+
+    // Offloaded experts (src/caif_device_frozen_linear.cpp:145-232): SetOffloadPolicy(HostPinned) and Evict()
+    // free a weight's device copy and Prefetch() uploads it to a new allocation.  The bank must refuse to run
+    // while an expert is away and must follow the weight to its new address afterwards.
+    typedef CAIF_OffloadPolicy::CAIF_OffloadPolicy_e Policy;
+    CAIF_DeviceFrozenLinearBase *moved=experts[2]->SubLayers().up.get();
+    moved->SetOffloadPolicy(Policy::HostPinned_e);
+    Report("bank forward with an evicted expert throws",Throws([&]{bank.Forward(x,off,false);},"Prefetch"));
+    // occupy the freed block so that the upload lands somewhere else
+    CAIF_DeviceTensor squatter=CAIF_DeviceTensor::Zeros({D,H},stream,Dtype_e::Int8);
+    moved->Prefetch(stream);
+    Report("bank forward after Prefetch equals the first result",Download(bank.Forward(x,off,true))==yb);
+    moved->Evict();
+    Report("bank backward with an evicted expert throws",Throws([&]{bank.Backward(g,off);},"Prefetch"));
+    moved->Prefetch(stream);
+    Report("bank backward after Prefetch equals the first result",Download(bank.Backward(g,off))==db);
+    moved->SetOffloadPolicy(Policy::GpuResident_e);
+    Report("bank forward after returning to GpuResident equals the first result",Download(bank.Forward(x,off,false))==yb);
   }
   stream.Synchronize();
 }

@@ -18,7 +18,7 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 from caif_amd import torch_ops as T                                  # noqa: E402
-from gpu_helpers import dev_as, host, make_weight, max_rel_err        # noqa: E402
+from gpu_helpers import dev, dev_as, host, make_weight, max_rel_err   # noqa: E402
 
 TOL_16 = 1e-2      # contract
 TOL_32 = 1e-4      # contract
@@ -152,3 +152,87 @@ def test_two_row_blocks_of_the_decode_kernel(orc, kind, M):
     # must come out of the second launch with the right offsets into X and Y
     _check(orc, np.random.default_rng(700 + M), M, 1536, 1024, kind, 2, 2)
     _check(orc, np.random.default_rng(701 + M), M, 200, 4096, kind, 1, 1, yd=2)
+
+
+@pytest.mark.parametrize("cd,xd", [(2, 0), (2, 1), (1, 0), (1, 2)])
+@pytest.mark.parametrize("K", [1024, 4096])
+@pytest.mark.parametrize("kind", ["int8pc", "int8pt"])
+def test_one_row_int8_casts_the_activations_to_the_compute_dtype(orc, kind, K, cd, xd):
+    # one activation row with int8 codes takes the integer-matrix-core kernel, which works on fp32 activations: when
+    # the caller's activations are of another type than the compute type they must pass through it first, as the
+    # layer's input.To(ComputeT) does (src/caif_device_frozen_linear.cpp:459).  fp32 activations that are not
+    # bf16 values make the difference visible: without the cast the error against the oracle is ~4e-3 here.
+    rng = np.random.default_rng(cd * 7 + xd + K)
+    ow, dw = make_weight(orc, rng, 2048, K, kind)
+    x = rng.normal(0, 1, (1, K)).astype(np.float32)
+    xt = dev_as(x, xd)
+    y = host(T.qlinear_forward(xt, dw, cd))
+    want = orc.frozen_linear_forward(host(xt), ow, cd)
+    assert max_rel_err(y, want) <= TIGHT_POST
+    # and an M = 1 call equals row 0 of an M = 16 call of the same accuracy class to fp32 rounding
+    x16 = dev_as(np.concatenate([x, rng.normal(0, 1, (15, K)).astype(np.float32)]), xd)
+    y16 = host(T.qlinear_forward(x16, dw, cd))
+    assert np.abs(y16[0] - y[0]).max() <= 2e-4 * np.abs(y16[0]).max()
+
+
+@pytest.mark.parametrize("kind", ["int8pc", "int8pt", "int4"])
+@pytest.mark.parametrize("M", [1, 2, 4, 16, 24])
+def test_non_finite_activations_are_not_masked(orc, kind, M):
+    # A NaN or an infinity in an activation row reaches every output of that row in the reference (dequantise +
+    # GEMM: every output multiplies every activation, and 0 * inf is NaN too).  The integer-matrix-core kernels
+    # split activations into digits, which has no meaning for such values: they must still answer non-finite for
+    # exactly those rows, and leave the other rows alone.
+    rng = np.random.default_rng(900 + M)
+    N, K = 1792, 4096
+    ow, dw = make_weight(orc, rng, N, K, kind)
+    for bad_value in (np.nan, np.inf, -np.inf):
+        x = rng.normal(0, 1, (M, K)).astype(np.float32)
+        bad_row = M - 1
+        x[bad_row, 1234] = bad_value
+        xt = dev_as(x, 2)
+        y = host(T.qlinear_forward(xt, dw, 2))
+        want = orc.frozen_linear_forward(host(xt), ow, 2)
+        assert not np.isfinite(want[bad_row]).any(), "the oracle's own answer for the poisoned row"
+        assert not np.isfinite(y[bad_row]).any(), (kind, M, bad_value)
+        good = [m for m in range(M) if m != bad_row]
+        if good:
+            assert np.isfinite(y[good]).all(), (kind, M, bad_value)
+            assert max_rel_err(y[good], want[good]) <= TIGHT_POST, (kind, M, bad_value)
+
+
+@pytest.mark.parametrize("kind", ["int4", "int8pc"])
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_post_scaled_kernels_on_correlated_inputs(orc, kind, M):
+    # The memory-bound kernels skip the reference's rounding of code*scale to bf16.  On N(0,1) activations those
+    # rounding differences add up like a random walk (about 2e-3 of max|ref|).  Correlated inputs are the worst
+    # case for that argument: all-positive activations against constant codes make every difference push the
+    # same way.  Cases: |N(0,1)| activations; alternating-sign constant activations; a weight whose every group
+    # holds one repeated code (so every product in a group shares one rounding difference); all-ones
+    # activations against that weight.  The contract's 1e-2 must hold on each; the worst value is recorded in the
+    # assertion message of the bound below.
+    rng = np.random.default_rng(77 + M)
+    N, K = 1792, 4096
+    cases = {}
+    w_rand = rng.normal(0, 0.02, (N, K)).astype(np.float32)
+    # constant code per 128-k group: each group's value is drawn once, so code*scale repeats 128 times
+    w_const = np.repeat(rng.normal(0, 0.02, (N, K // 128)).astype(np.float32), 128, axis=1)
+    x_abs = np.abs(rng.normal(0, 1, (M, K))).astype(np.float32)
+    x_alt = np.tile(np.array([1.0, -1.0], np.float32), (M, K // 2)) * 0.7311
+    x_one = np.ones((M, K), np.float32)
+    for wname, w in (("random", w_rand), ("constant-per-group", w_const)):
+        if kind == "int4":
+            p, s = orc.quantize_to_int4(w, 128)
+            ow = orc.FrozenWeight(p, orc.W_INT4_GROUP, s, N, K, 1, 128)
+            dw = T.FrozenWeight(dev(p), T.W_INT4_GROUP, dev(s.view(np.float16)), N, K, 1, 128)
+        else:
+            q, s = orc.quantize_int8_per_channel(w.reshape(K, N))
+            ow = orc.FrozenWeight(q.reshape(-1), orc.W_INT8, s, N, K, N, 128)
+            dw = T.FrozenWeight(dev(q.reshape(-1)), T.W_INT8, dev(s), N, K, N, 128)
+        for xname, x in (("abs-normal", x_abs), ("alternating", x_alt), ("ones", x_one)):
+            xt = dev_as(x, 2)
+            y = host(T.qlinear_forward(xt, dw, 2))
+            want = orc.frozen_linear_forward(host(xt), ow, 2)
+            cases[(wname, xname)] = max_rel_err(y, want)
+    worst = max(cases.values())
+    print(f"post-scaled {kind} M={M}: " + ", ".join(f"{w}/{x}={e:.2e}" for (w, x), e in cases.items()))
+    assert worst <= TOL_16, cases

@@ -194,3 +194,61 @@ def test_dispatch_map_is_a_bijection_onto_segments(orc):
     flat_e = idx.ravel()
     for e in range(E):
         assert np.array_equal(dmap.ravel()[flat_e == e], np.arange((flat_e == e).sum()))
+
+
+# --------------------------------------------------------------------------- LoRA wrapper around the frozen base
+def _lora_case(orc, seed, kind, M=7, N=24, K=32, rank=4):
+    rng = np.random.default_rng(seed)
+    fw, _ = _w(orc, rng, N, K, kind)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    g = rng.normal(0, 1e-3, (M, N)).astype(np.float32)
+    a = rng.normal(0, 0.01, (rank, K)).astype(np.float32)
+    b = rng.normal(0, 0.01, (N, rank)).astype(np.float32)
+    return fw, x, g, a, b
+
+
+@pytest.mark.parametrize("kind", ["int4", "int8pc"])
+def test_lora_forward_and_input_gradient_against_float64_composition(orc, kind):
+    # out = x W^T + (alpha/rank) (x A^T) B^T and dX = g W + (alpha/rank) (g B) A
+    # (src/caif_device_lora_adapter.cpp:161-198, 228-276), written here with numpy float64 matmuls on the
+    # materialised weight.  With fp32 storage and compute the oracle's intermediate casts are identities, so it
+    # must agree to fp32 rounding; with bf16 it must agree to the size of its seven bf16 roundings.
+    alpha, rank = 32.0, 4
+    fw, x, g, a, b = _lora_case(orc, 31, kind)
+    W = fw.compute_weight(0).astype(np.float64)
+    x64, g64, a64, b64 = (v.astype(np.float64) for v in (x, g, a, b))
+    want_y = x64 @ W.T + (alpha / rank) * (x64 @ a64.T) @ b64.T
+    want_dx = g64 @ W + (alpha / rank) * (g64 @ b64) @ a64
+    y, hidden = orc.lora_forward(x, fw, a, b, alpha, 0, 0)
+    dx = orc.lora_backward_input(g, fw, a, b, alpha, 0, 0)
+    assert np.abs(y - want_y).max() <= 1e-5 * np.abs(want_y).max()
+    assert np.abs(hidden - x64 @ a64.T).max() <= 1e-5 * np.abs(x64 @ a64.T).max()
+    assert np.abs(dx - want_dx).max() <= 1e-5 * np.abs(want_dx).max()
+    # a swapped operand or a dropped alpha/rank would be off by far more than this
+    wrong_y = x64 @ W.T + (x64 @ a64.T) @ b64.T
+    assert np.abs(y - wrong_y).max() > 1e-3 * np.abs(want_y).max()
+    # bf16 storage and compute: the same quantities, each intermediate rounded to 8 bits of mantissa
+    xb = orc.round_to_dtype(x, 2)
+    gb = orc.round_to_dtype(g, 2)
+    yb, _ = orc.lora_forward(xb, fw, a, b, alpha, 2, 2)
+    dxb = orc.lora_backward_input(gb, fw, a, b, alpha, 2, 2)
+    Wb = fw.compute_weight(2).astype(np.float64)
+    ab, bb = orc.round_to_dtype(a, 2).astype(np.float64), orc.round_to_dtype(b, 2).astype(np.float64)
+    want_yb = xb.astype(np.float64) @ Wb.T + (alpha / rank) * (xb.astype(np.float64) @ ab.T) @ bb.T
+    want_dxb = gb.astype(np.float64) @ Wb + (alpha / rank) * (gb.astype(np.float64) @ bb) @ ab
+    assert np.abs(yb - want_yb).max() <= 2e-2 * np.abs(want_yb).max()
+    assert np.abs(dxb - want_dxb).max() <= 2e-2 * np.abs(want_dxb).max()
+
+
+@pytest.mark.parametrize("sd", [0, 1, 2])
+def test_lora_with_zero_b_is_the_base_layer(orc, sd):
+    # B = 0 is how every adapter starts (tests/test_device_lora_adapter.cpp:371-443): the low-rank branch adds an
+    # exact zero, so output and input gradient are the base layer's, cast to the storage dtype
+    fw, x, g, a, b = _lora_case(orc, 32, "int4")
+    b[:] = 0.0
+    cd = sd
+    y, _ = orc.lora_forward(x, fw, a, b, 32.0, cd, sd)
+    dx = orc.lora_backward_input(g, fw, a, b, 32.0, cd, sd)
+    xs, gs = orc.round_to_dtype(x, sd), orc.round_to_dtype(g, sd)
+    assert np.array_equal(y, orc.round_to_dtype(orc.frozen_linear_forward(xs, fw, cd), sd))
+    assert np.array_equal(dx, orc.round_to_dtype(orc.frozen_linear_backward(gs, fw, cd), sd))
