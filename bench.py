@@ -46,6 +46,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--replays", type=int, default=5,
+                    help="the K-step timed region is run this many times; the median run is reported")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary rows (M=4/16, GEMM TFLOP/s)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -124,11 +126,17 @@ def main():
     graph = capture(step, args.steps)
     graph.replay()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    graph.replay()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    # exactly K steps per timed run, each run bracketed by a device synchronisation on both sides; one run of a
+    # 20-step graph lasts well under a millisecond, so the median of several runs is what is reported
+    runs_ms = []
+    for _ in range(max(1, args.replays)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        runs_ms.append((t1 - t0) * 1e3 / args.steps)
+    ms_per_step = sorted(runs_ms)[len(runs_ms) // 2]
     step_bytes = algorithmic_bytes("int4", 1) + algorithmic_bytes("int8", 1)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
@@ -180,12 +188,17 @@ def main():
         "decode_cache_resident_GBps_M1": {k: round(v, 1) for k, v in resident.items()},
         "decode_frac_of_hbm_peak_M1": {k: round(per[(k, 1)]["GBps"] / HBM_PEAK_GBS, 4) for k in ("int4", "int8")},
         "weight_copies_rotated": {"int4": copies4, "int8": copies8},
+        "timed_runs_ms_per_step": [round(v, 6) for v in runs_ms],
     }
     if not args.no_extra:
-        try:
-            extra.update(compute_bound_rows(torch, T, dev, gen, capture, time_graph))
-        except Exception as e:   # secondary rows must not take the headline down
-            extra["compute_bound_error"] = repr(e)
+        del W4[1:], W8[1:]                        # the rotated copies are not needed below
+        for name, fn in (("decode_other_shapes", lambda: decode_other_rows(torch, T, dev, gen, capture, time_graph)),
+                         ("quantise_ops", lambda: quantise_rows(torch, T, dev, gen)),
+                         ("compute_bound", lambda: compute_bound_rows(torch, T, dev, gen, capture, time_graph))):
+            try:
+                extra.update(fn())
+            except Exception as e:   # secondary rows must not take the headline down
+                extra[name + "_error"] = repr(e)
 
     out = {
         "metric": "dequant-GEMM HBM GB/s (M=1 int4/int8) + MFMA TFLOP/s (M=2048 fwd+dX)",
@@ -210,7 +223,98 @@ def main():
         out["cpu_baseline"] = cpu_baseline(np, q8.cpu().numpy(), s8.cpu().numpy(), p4.cpu().numpy(),
                                            s4.cpu().view(torch.int16).numpy().view(np.uint16),
                                            X[1].float().cpu().numpy())
+        if not args.no_extra:
+            extra["cpu_host_path_configs0"] = cpu_configs0(np)
     print(json.dumps(out))
+
+
+def decode_other_rows(torch, T, dev, gen, capture, time_graph):
+    """Decode launches beside the headline shape.
+    `decode_tall_M1`: the same M = 1 kernels on a weight eight times as tall (N = 114688, K = 4096; 235 MB int4,
+    470 MB int8, and successive launches read different copies): one launch streams long enough that its start
+    and end no longer weigh, so the rate it reaches is the kernels' streaming rate and the distance of the N = 14336 launches
+    from it is what a launch's ramp and tail cost.
+    `decode_down_proj`: the FFN down projection of the same model (N = 4096, K = 14336), M = 1 and 16."""
+    out = {"decode_tall_M1": {}, "decode_down_proj": {}}
+    x1 = torch.empty(1, K_DEC, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16)
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    N_TALL = 8 * N_DEC
+    w = torch.empty(N_TALL, K_DEC, device=dev).normal_(0, 0.02, generator=gen)
+    p4, s4 = T.quantize_int4_per_group(w, 128)
+    q8, s8 = T.quantize_int8(w.reshape(K_DEC, N_TALL), per_channel=True)
+    del w
+    y = torch.empty(1, N_TALL, device=dev)
+    # each launch reads a different copy, and the copies together exceed 512 MB, so none of it comes from cache
+    tall = (("int4", [T.FrozenWeight(p4.clone() if i else p4, T.W_INT4_GROUP, s4, N_TALL, K_DEC, 1, 128)
+                      for i in range(3)]),
+            ("int8", [T.FrozenWeight(q8.reshape(-1).clone() if i else q8.reshape(-1), T.W_INT8, s8, N_TALL, K_DEC,
+                                     N_TALL) for i in range(2)]))
+    for kind, fws in tall:
+        g = capture(lambda i, fws=fws: T.qlinear_forward(x1, fws[i % len(fws)], T.BF16, T.F32, out=y, workspace=ws),
+                    12)
+        ms = time_graph(g, 12)
+        del g
+        nbytes = algorithmic_bytes(kind, 1, N=N_TALL)
+        out["decode_tall_M1"][kind] = {"N": N_TALL, "copies_rotated": len(fws), "us": round(ms * 1e3, 2),
+                                       "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                       "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    del tall, fws
+    del p4, s4, q8, s8, y
+    N, K = 4096, 14336
+    copies = 10                                  # 10 x 59 MB (int8) / 20 x 30 MB (int4) > 512 MB: HBM, not cache
+    w = torch.empty(N, K, device=dev).normal_(0, 0.02, generator=gen)
+    p4, s4 = T.quantize_int4_per_group(w, 128)
+    q8, s8 = T.quantize_int8(w.reshape(K, N), per_channel=True)
+    del w
+    W4 = [T.FrozenWeight(p4.clone(), T.W_INT4_GROUP, s4, N, K, 1, 128) for _ in range(2 * copies)]
+    W8 = [T.FrozenWeight(q8.reshape(-1).clone(), T.W_INT8, s8, N, K, N) for _ in range(copies)]
+    for m in (1, 16):
+        x = torch.empty(m, K, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16)
+        y = torch.empty(m, N, device=dev)
+        for kind, Ws in (("int4", W4), ("int8", W8)):
+            g = capture(lambda i, Ws=Ws: T.qlinear_forward(x, Ws[i % len(Ws)], T.BF16, T.F32, out=y, workspace=ws), 40)
+            ms = time_graph(g, 40)
+            del g
+            nbytes = algorithmic_bytes(kind, m, N=N, K=K)
+            out["decode_down_proj"][f"{kind}_M{m}_N{N}_K{K}"] = {
+                "us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    return out
+
+
+def quantise_rows(torch, T, dev, gen):
+    """The quantise / pack ops on the decode weight (fp32 [4096, 14336], 235 MB): eager calls timed with HIP
+    events.  Bytes counted: one read of the input plus the codes and scales written; the int8 schemes need the
+    maxima before the first code, so a second read of an input this size (larger than the caches) is part of
+    their cost and shows as a lower fraction."""
+    rows, cols = K_DEC, N_DEC
+    w = torch.empty(rows, cols, device=dev).normal_(0, 0.02, generator=gen)
+    n = rows * cols
+    out = {}
+
+    def timed(fn, iters=10):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) / iters)
+        return sorted(ts)[1]
+
+    for name, fn, nbytes in (
+            ("int8_per_channel_4096x14336", lambda: T.quantize_int8(w, per_channel=True), n * 4 + n + cols * 4),
+            ("int8_per_tensor_4096x14336", lambda: T.quantize_int8(w, per_channel=False), n * 4 + n + 4),
+            ("int4_group128_4096x14336", lambda: T.quantize_int4_per_group(w, 128), n * 4 + n // 2 + n // 128 * 2)):
+        ms = timed(fn)
+        out[name] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                     "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    return {"quantise_ops": out}
 
 
 def compute_bound_rows(torch, T, dev, gen, capture, time_graph):
@@ -326,6 +430,13 @@ def fp32_rows(torch, T, dev, gen, capture, time_graph):
             "fwd_us": round(ms_f * 1e3, 2), "dx_us": round(ms_b * 1e3, 2),
             "fwd_TFLOPs": round(flops / (ms_f * 1e-3) / 1e12, 2), "dx_TFLOPs": round(flops / (ms_b * 1e-3) / 1e12, 2),
             "fwd_dx_frac_of_fp32_mfma_peak": round(2 * flops / ((ms_f + ms_b) * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4)}
+        if M == 16:
+            # sixteen rows against a 16.8 MB weight: the weight stream bounds it, not the matrix pipes
+            nbytes = N * K + N * 4 + M * K * 4 + M * N * 4
+            rows[f"int8_M{M}_N{N}_K{K}"].update({
+                "bound": "hbm", "algorithmic_bytes": nbytes,
+                "fwd_frac_of_hbm_peak": round(nbytes / (ms_f * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                "dx_frac_of_hbm_peak": round(nbytes / (ms_b * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
     return rows
 
 
@@ -425,17 +536,6 @@ def moe_rows(torch, T, dev, gen):
             routing[name].update({"GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                   "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
     routing_ms = sum(v["us"] for v in routing.values()) * 1e-3
-    # per-expert-segment efficiency: replay single segments (shortest, median, longest) of the gate
-    # projection as stand-alone dequant-GEMMs
-    order = torch.argsort(counts).tolist()
-    segments = {}
-    for label, e in (("shortest", order[0]), ("median", order[E // 2]), ("longest", order[-1])):
-        lo, hi = int(offsets[e]), int(offsets[e + 1])
-        xe, ye = x[lo:hi], up_o[lo:hi]
-        ms = timed(lambda: T.qlinear_forward(xe, gate.weights[e], T.BF16, T.BF16, out=ye, workspace=ws), iters=20)
-        fl = 2.0 * (hi - lo) * D * H
-        segments[label] = {"rows": hi - lo, "us": round(ms * 1e3, 2), "TFLOPs": round(fl / (ms * 1e-3) / 1e12, 1),
-                           "frac_of_mfma_peak": round(fl / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
     gemm_flops = 3 * 2.0 * rows * D * H
     return {"experts": E, "tokens": tokens, "top_k": top_k, "packed_rows": rows,
             "rows_per_expert_min_max": [int(counts.min()), int(counts.max())],
@@ -449,8 +549,7 @@ def moe_rows(torch, T, dev, gen):
             # the other bound of a pass: every expert weight (int8 codes + fp32 per-channel scales) streamed once
             "weight_bytes_per_pass": int(3 * E * D * H + E * (2 * H + D) * 4),
             "weight_stream_us_at_hbm_peak": round((3 * E * D * H + E * (2 * H + D) * 4) / (HBM_PEAK_GBS * 1e9) * 1e6, 1),
-            "mfma_us_at_peak_per_pass": round(gemm_flops / (MFMA_BF16_PEAK_TFLOPS * 1e12) * 1e6, 1),
-            "single_segment_replay_gate_proj": segments}
+            "mfma_us_at_peak_per_pass": round(gemm_flops / (MFMA_BF16_PEAK_TFLOPS * 1e12) * 1e6, 1)}
 
 
 def cpu_baseline(np, q8, s8, p4, s4_bits, x_values):
@@ -460,7 +559,8 @@ def cpu_baseline(np, q8, s8, p4, s4_bits, x_values):
     same M=1 workload.  Bounded: at most ~20 s of CPU work."""
     from oracle import oracle as orc
     orc.build()
-    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    omp_threads, blas_threads = cpu_threads(orc)
+    cores = max(omp_threads, blas_threads)
     x = np.ascontiguousarray(x_values, np.float32)
     reps, t_deq, t_gemm = 0, 0.0, 0.0
     t_start = time.perf_counter()
@@ -484,10 +584,53 @@ def cpu_baseline(np, q8, s8, p4, s4_bits, x_values):
         "cores": cores,
         "kind": "port",
         "sample": f"{reps} full steps of the same M=1 workload (int4 + int8, K=4096, N=14336): oracle OpenMP "
-                  f"dequantise-to-fp32 ({t_deq / reps * 1e3:.1f} ms/step) + numpy/OpenBLAS sgemm "
-                  f"({t_gemm / reps * 1e3:.1f} ms/step)",
+                  f"dequantise-to-fp32 ({t_deq / reps * 1e3:.1f} ms/step, {omp_threads} OpenMP threads) + "
+                  f"numpy/OpenBLAS sgemm ({t_gemm / reps * 1e3:.1f} ms/step, {blas_threads} OpenBLAS threads)",
         "ms_per_step": round(per_step * 1e3, 3),
     }
+
+
+def cpu_threads(orc):
+    """(OpenMP threads of the oracle's loops, threads of numpy's BLAS) as the libraries themselves report them."""
+    blas = 1
+    try:
+        from threadpoolctl import threadpool_info
+        blas = max([p.get("num_threads", 1) for p in threadpool_info() if p.get("user_api") == "blas"] or [1])
+    except Exception:
+        pass
+    return orc.max_threads(), blas
+
+
+def cpu_configs0(np):
+    """BASELINE configs[0] on the host cores: the reference's Host_e path is cblas_sgemm on an fp32 weight
+    (src/caif_ops_host.cpp:54-139), forward (NoTrans, Trans) and input gradient (NoTrans, NoTrans); the weight is
+    the oracle's dequantised int8 per-channel weight (dequantisation timed separately, the reference has no host
+    dequantiser).  K = N = 4096, fp32 X[16, 4096] ~ N(0,1), dY ~ N(0, 1e-3)."""
+    from oracle import oracle as orc
+    orc.build()
+    rng = np.random.default_rng(7)
+    N = K = 4096
+    w = rng.normal(0, 0.02, (K, N)).astype(np.float32)
+    q, s = orc.quantize_int8_per_channel(w)
+    x = rng.normal(0, 1, (16, K)).astype(np.float32)
+    dy = rng.normal(0, 1e-3, (16, N)).astype(np.float32)
+    t0 = time.perf_counter()
+    wf = orc.frozen_weight_compute(q.reshape(-1), orc.W_INT8, s, N, K, N, 128, orc.F32)
+    t_deq = time.perf_counter() - t0
+    fwd, bwd = [], []
+    for _ in range(7):
+        t0 = time.perf_counter()
+        y = x @ wf.T
+        t1 = time.perf_counter()
+        dx = dy @ wf
+        t2 = time.perf_counter()
+        fwd.append(t1 - t0)
+        bwd.append(t2 - t1)
+    del y, dx
+    omp_threads, blas_threads = cpu_threads(orc)
+    return {"workload": "int8 per-channel K=N=4096, fp32 X[16,4096]: sgemm forward + input gradient on the dequantised weight",
+            "dequantise_ms": round(t_deq * 1e3, 2), "sgemm_fwd_ms": round(sorted(fwd)[3] * 1e3, 3),
+            "sgemm_dx_ms": round(sorted(bwd)[3] * 1e3, 3), "openmp_threads": omp_threads, "openblas_threads": blas_threads}
 
 
 if __name__ == "__main__":

@@ -24,7 +24,21 @@
 #include <stdlib.h>
 #include <string.h>
 
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
 #define ORC_API __attribute__((visibility("default")))
+
+/* threads the parallel loops below run on (what a timed CPU baseline has to state) */
+ORC_API int orc_max_threads(void)
+{
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
 
 /* dtype codes shared with include/caifx.h */
 enum { ORC_F32 = 0, ORC_F16 = 1, ORC_BF16 = 2 };

@@ -51,6 +51,13 @@ _i64, _i32, _u32 = ctypes.c_int64, ctypes.c_int32, ctypes.c_uint32
 _p = ctypes.c_void_p
 
 
+def max_threads():
+    """OpenMP threads the oracle's parallel loops use."""
+    L = lib()
+    L.orc_max_threads.restype = ctypes.c_int
+    return int(L.orc_max_threads())
+
+
 def _declare(L):
     L.orc_f32_to_bf16.restype = ctypes.c_uint16
     L.orc_f32_to_bf16.argtypes = [ctypes.c_float]
