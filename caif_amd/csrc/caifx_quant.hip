@@ -70,14 +70,40 @@ __global__ void fill_u32_kernel(uint32_t *p, int64_t n, uint32_t v)
 
 // max |x| over the whole tensor -> atomicMax on the bit pattern (non-negative floats order
 // like unsigned integers).  `v > m` drops NaNs exactly like the reference's comparison.
-__global__ void absmax_tensor_kernel(const float *__restrict__ in, uint32_t *__restrict__ acc, int64_t n)
+// `vec`: the input is 16-byte aligned, so the body goes in 16-byte loads (four of them in flight per lane) and
+// the last n % 4 elements are left to the first lanes.
+__global__ void absmax_tensor_kernel(const float *__restrict__ in, uint32_t *__restrict__ acc, int64_t n, int vec)
 {
   __shared__ float part[kBlock / kWave];
   float m = 0.0f;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
-    float v = fabsf(in[i]);
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  auto take = [&](float v) {
+    v = fabsf(v);
     if (v > m) m = v;
+  };
+  if (vec) {
+    const floatx4_t *in4 = reinterpret_cast<const floatx4_t *>(in);
+    const int64_t n4 = n >> 2;
+    int64_t i = first;
+    for (; i + 3 * stride < n4; i += 4 * stride) {
+      const floatx4_t a = in4[i], b = in4[i + stride], c = in4[i + 2 * stride], d = in4[i + 3 * stride];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        take(a[j]);
+        take(b[j]);
+        take(c[j]);
+        take(d[j]);
+      }
+    }
+    for (; i < n4; i += stride) {
+      const floatx4_t a = in4[i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) take(a[j]);
+    }
+    if (first < (n & 3)) take(in[(n4 << 2) + first]);
+  } else {
+    for (int64_t i = first; i < n; i += stride) take(in[i]);
   }
   m = wave_max(m);
   if ((threadIdx.x & (kWave - 1)) == 0) part[threadIdx.x / kWave] = m;
@@ -105,6 +131,40 @@ __global__ void absmax_columns_kernel(const float *__restrict__ in, uint32_t *__
   if (m > 0.0f) atomicMax(acc + c, __float_as_uint(m));
 }
 
+// The same with four adjacent columns per thread (cols % 4 == 0, 16-byte aligned input): 16-byte loads, four
+// rows in flight per lane.
+__global__ void absmax_columns_x4_kernel(const float *__restrict__ in, uint32_t *__restrict__ acc, int rows, int cols)
+{
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (c >= cols) return;
+  const int r0 = blockIdx.y * kRowChunk;
+  const int r1 = r0 + kRowChunk < rows ? r0 + kRowChunk : rows;
+  float m[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  const float *p = in + static_cast<int64_t>(r0) * cols + c;
+  auto take = [&](const floatx4_t &v) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float a = fabsf(v[j]);
+      if (a > m[j]) m[j] = a;
+    }
+  };
+  int r = r0;
+  for (; r + 4 <= r1; r += 4, p += 4 * static_cast<int64_t>(cols)) {
+    const floatx4_t a = *reinterpret_cast<const floatx4_t *>(p);
+    const floatx4_t b = *reinterpret_cast<const floatx4_t *>(p + cols);
+    const floatx4_t d = *reinterpret_cast<const floatx4_t *>(p + 2 * static_cast<int64_t>(cols));
+    const floatx4_t e = *reinterpret_cast<const floatx4_t *>(p + 3 * static_cast<int64_t>(cols));
+    take(a);
+    take(b);
+    take(d);
+    take(e);
+  }
+  for (; r < r1; ++r, p += cols) take(*reinterpret_cast<const floatx4_t *>(p));
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    if (m[j] > 0.0f) atomicMax(acc + c + j, __float_as_uint(m[j]));
+}
+
 // in place: max|x| -> scale = max / 127 (1.0 when max is zero)
 __global__ void finalize_int8_scale_kernel(float *scales, int count)
 {
@@ -130,6 +190,68 @@ __global__ void quantize_int8_kernel(const float *__restrict__ in, int8_t *__res
   }
 }
 
+__device__ __forceinline__ uint32_t quantize_int8_x4(const floatx4_t &v, const float (&inv)[4])
+{
+  uint32_t w = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    w |= (static_cast<uint32_t>(static_cast<int>(rintf(clamp_sym(v[j] * inv[j], kInt8Max)))) & 0xFFu) << (8 * j);
+  return w;
+}
+
+// One scale for the whole tensor, 16 consecutive elements per thread (16-byte aligned input and output,
+// n % 16 == 0): same arithmetic per element as quantize_int8_kernel, the reciprocal taken once per thread.
+__global__ void quantize_int8_tensor_x16_kernel(const float *__restrict__ in, int8_t *__restrict__ out,
+                                                const float *__restrict__ scale, int64_t n16)
+{
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n16) return;
+  const float s = scale[0];
+  const float one = (s > 0.0f) ? 1.0f / s : 0.0f;
+  const float inv[4] = {one, one, one, one};
+  const floatx4_t *p = reinterpret_cast<const floatx4_t *>(in) + i * 4;
+  const floatx4_t a = p[0], b = p[1], c = p[2], d = p[3];
+  u32x4_t w;
+  w[0] = quantize_int8_x4(a, inv);
+  w[1] = quantize_int8_x4(b, inv);
+  w[2] = quantize_int8_x4(c, inv);
+  w[3] = quantize_int8_x4(d, inv);
+  reinterpret_cast<u32x4_t *>(out)[i] = w;
+}
+
+// One scale per column of a [rows, cols] tensor: a thread takes four adjacent columns (cols % 4 == 0, aligned
+// pointers) and kQuantRows consecutive rows, so the four reciprocals are taken once for all of them.  The row
+// blocks are walked from the last to the first: the maxima pass before this one read the tensor front to back,
+// so its tail is what the caches still hold.
+constexpr int kQuantRows = 16;
+__global__ void quantize_int8_columns_x4_kernel(const float *__restrict__ in, int8_t *__restrict__ out,
+                                                const float *__restrict__ scales, int rows, int cols)
+{
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (c >= cols) return;
+  const int r0 = (gridDim.y - 1 - blockIdx.y) * kQuantRows;
+  const int r1 = r0 + kQuantRows < rows ? r0 + kQuantRows : rows;
+  const floatx4_t s = *reinterpret_cast<const floatx4_t *>(scales + c);
+  float inv[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) inv[j] = (s[j] > 0.0f) ? 1.0f / s[j] : 0.0f;
+  const float *p = in + static_cast<int64_t>(r0) * cols + c;
+  int8_t *q = out + static_cast<int64_t>(r0) * cols + c;
+  int r = r0;
+  for (; r + 4 <= r1; r += 4, p += 4 * static_cast<int64_t>(cols), q += 4 * static_cast<int64_t>(cols)) {
+    const floatx4_t a = *reinterpret_cast<const floatx4_t *>(p);
+    const floatx4_t b = *reinterpret_cast<const floatx4_t *>(p + cols);
+    const floatx4_t d = *reinterpret_cast<const floatx4_t *>(p + 2 * static_cast<int64_t>(cols));
+    const floatx4_t e = *reinterpret_cast<const floatx4_t *>(p + 3 * static_cast<int64_t>(cols));
+    *reinterpret_cast<uint32_t *>(q) = quantize_int8_x4(a, inv);
+    *reinterpret_cast<uint32_t *>(q + cols) = quantize_int8_x4(b, inv);
+    *reinterpret_cast<uint32_t *>(q + 2 * static_cast<int64_t>(cols)) = quantize_int8_x4(d, inv);
+    *reinterpret_cast<uint32_t *>(q + 3 * static_cast<int64_t>(cols)) = quantize_int8_x4(e, inv);
+  }
+  for (; r < r1; ++r, p += cols, q += cols)
+    *reinterpret_cast<uint32_t *>(q) = quantize_int8_x4(*reinterpret_cast<const floatx4_t *>(p), inv);
+}
+
 __global__ void dequantize_int8_kernel(const int8_t *__restrict__ in, float *__restrict__ out,
                                        const float *__restrict__ scales, int64_t n, int period)
 {
@@ -146,15 +268,26 @@ __global__ void dequantize_int8_kernel(const int8_t *__restrict__ in, float *__r
 // ------------------------------------------------------------------ int4 per-group
 // Fast path: each thread owns 8 consecutive elements (one dword of packed output); a team of
 // group_size/8 adjacent lanes owns one group and shares its max through wave shuffles.
-// Needs group_size % 8 == 0 and group_size/8 a power of two <= 64.
+// Needs group_size % 8 == 0 and group_size/8 a power of two <= 64.  `vec`: the input is 16-byte aligned (two
+// 16-byte loads per thread).
 __global__ void quantize_int4_team_kernel(const float *__restrict__ in, uint8_t *__restrict__ packed,
-                                          f16_t *__restrict__ scales, int64_t n, int group_size, int team)
+                                          f16_t *__restrict__ scales, int64_t n, int group_size, int team, int vec)
 {
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const int64_t base = gid * 8;
   float x[8];
+  if (vec && base + 8 <= n) {
+    const floatx4_t lo = *reinterpret_cast<const floatx4_t *>(in + base);
+    const floatx4_t hi = *reinterpret_cast<const floatx4_t *>(in + base + 4);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) x[j] = (base + j < n) ? in[base + j] : 0.0f;
+    for (int j = 0; j < 4; ++j) {
+      x[j] = lo[j];
+      x[4 + j] = hi[j];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = (base + j < n) ? in[base + j] : 0.0f;
+  }
   float m = 0.0f;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
@@ -212,15 +345,23 @@ __global__ void quantize_int4_serial_kernel(const float *__restrict__ in, uint8_
 
 // out[f] = float(code) * float(scale[f / group]); 8 elements (one packed dword) per thread
 __global__ void dequantize_int4_x8_kernel(const uint8_t *__restrict__ packed, const f16_t *__restrict__ scales,
-                                          float *__restrict__ out, int64_t n, int group_size)
+                                          float *__restrict__ out, int64_t n, int group_size, int vec)
 {
   const int64_t base = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 8;
   if (base >= n) return;
   if (base + 8 <= n) {
     const uint32_t w = *reinterpret_cast<const uint32_t *>(packed + base / 2);
     const float s = static_cast<float>(scales[base / group_size]);
+    float e[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) out[base + j] = static_cast<float>(nibble_s4(w >> (4 * j), 0)) * s;
+    for (int j = 0; j < 8; ++j) e[j] = static_cast<float>(nibble_s4(w >> (4 * j), 0)) * s;
+    if (vec) {
+      *reinterpret_cast<floatx4_t *>(out + base) = floatx4_t{e[0], e[1], e[2], e[3]};
+      *reinterpret_cast<floatx4_t *>(out + base + 4) = floatx4_t{e[4], e[5], e[6], e[7]};
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) out[base + j] = e[j];
+    }
   } else {
     for (int64_t f = base; f < n; ++f) {
       const uint32_t b = packed[f / 2];
@@ -285,10 +426,16 @@ int caifx_quantize_int8_per_tensor(const float *input, void *output, void *scale
   hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, s, static_cast<uint32_t *>(scale), int64_t{1}, 0u);
   int blocks = grid_for(n);
   if (blocks > 2048) blocks = 2048;
-  hipLaunchKernelGGL(absmax_tensor_kernel, dim3(blocks), dim3(kBlock), 0, s, input, static_cast<uint32_t *>(scale), n);
+  hipLaunchKernelGGL(absmax_tensor_kernel, dim3(blocks), dim3(kBlock), 0, s, input, static_cast<uint32_t *>(scale), n,
+                     aligned_to(input, 16) ? 1 : 0);
   hipLaunchKernelGGL(finalize_int8_scale_kernel, dim3(1), dim3(64), 0, s, static_cast<float *>(scale), 1);
-  hipLaunchKernelGGL(quantize_int8_kernel, dim3(grid_for((n + 3) / 4)), dim3(kBlock), 0, s, input,
-                     static_cast<int8_t *>(output), static_cast<const float *>(scale), n, 1);
+  const int64_t body = (aligned_to(input, 16) && aligned_to(output, 16)) ? n / 16 * 16 : 0;
+  if (body > 0)
+    hipLaunchKernelGGL(quantize_int8_tensor_x16_kernel, dim3(grid_for(body / 16)), dim3(kBlock), 0, s, input,
+                       static_cast<int8_t *>(output), static_cast<const float *>(scale), body / 16);
+  if (body < n)
+    hipLaunchKernelGGL(quantize_int8_kernel, dim3(grid_for((n - body + 3) / 4)), dim3(kBlock), 0, s, input + body,
+                       static_cast<int8_t *>(output) + body, static_cast<const float *>(scale), n - body, 1);
   return launch_status();
 }
 
@@ -312,12 +459,24 @@ int caifx_quantize_int8_per_channel(const float *input, void *output, void *scal
   const int64_t n = static_cast<int64_t>(rows) * cols;
   hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(cols)), dim3(kBlock), 0, s, static_cast<uint32_t *>(scales),
                      static_cast<int64_t>(cols), 0u);
-  hipLaunchKernelGGL(absmax_columns_kernel, dim3(grid_for(cols), (rows + kRowChunk - 1) / kRowChunk), dim3(kBlock), 0, s,
-                     input, static_cast<uint32_t *>(scales), rows, cols);
+  // four columns per thread when every row starts 16-byte aligned (and the codes of a row 4-byte aligned)
+  const bool x4 = cols % 4 == 0 && aligned_to(input, 16) && aligned_to(output, 4) && aligned_to(scales, 16) &&
+                  (rows + kQuantRows - 1) / kQuantRows <= 65535;
+  if (x4)
+    hipLaunchKernelGGL(absmax_columns_x4_kernel, dim3(grid_for(cols / 4, 64), (rows + kRowChunk - 1) / kRowChunk), dim3(64),
+                       0, s, input, static_cast<uint32_t *>(scales), rows, cols);
+  else
+    hipLaunchKernelGGL(absmax_columns_kernel, dim3(grid_for(cols), (rows + kRowChunk - 1) / kRowChunk), dim3(kBlock), 0,
+                       s, input, static_cast<uint32_t *>(scales), rows, cols);
   hipLaunchKernelGGL(finalize_int8_scale_kernel, dim3(grid_for(cols)), dim3(kBlock), 0, s,
                      static_cast<float *>(scales), cols);
-  hipLaunchKernelGGL(quantize_int8_kernel, dim3(grid_for((n + 3) / 4)), dim3(kBlock), 0, s, input,
-                     static_cast<int8_t *>(output), static_cast<const float *>(scales), n, cols);
+  if (x4)
+    hipLaunchKernelGGL(quantize_int8_columns_x4_kernel, dim3(grid_for(cols / 4, 64), (rows + kQuantRows - 1) / kQuantRows),
+                       dim3(64), 0, s, input, static_cast<int8_t *>(output), static_cast<const float *>(scales), rows,
+                       cols);
+  else
+    hipLaunchKernelGGL(quantize_int8_kernel, dim3(grid_for((n + 3) / 4)), dim3(kBlock), 0, s, input,
+                       static_cast<int8_t *>(output), static_cast<const float *>(scales), n, cols);
   return launch_status();
 }
 
@@ -347,7 +506,7 @@ int caifx_quantize_to_int4(const float *input, void *packed_output, void *scales
     const int64_t threads = (num_elements + 7) / 8;
     hipLaunchKernelGGL(quantize_int4_team_kernel, dim3(grid_for(threads)), dim3(kBlock), 0, s, input,
                        static_cast<uint8_t *>(packed_output), static_cast<f16_t *>(scales_output), num_elements,
-                       group_size, team);
+                       group_size, team, aligned_to(input, 16) ? 1 : 0);
   } else {
     const int64_t groups = (num_elements + group_size - 1) / group_size;
     hipLaunchKernelGGL(quantize_int4_serial_kernel, dim3(grid_for(groups)), dim3(kBlock), 0, s, input,
@@ -367,7 +526,7 @@ int caifx_dequantize_int4(const void *packed_data, const void *scales, float *ou
   if (group_size % 8 == 0 && aligned_to(packed_data, 4)) {
     hipLaunchKernelGGL(dequantize_int4_x8_kernel, dim3(grid_for((num_elements + 7) / 8)), dim3(kBlock), 0, s,
                        static_cast<const uint8_t *>(packed_data), static_cast<const f16_t *>(scales), output,
-                       num_elements, group_size);
+                       num_elements, group_size, aligned_to(output, 16) ? 1 : 0);
   } else {
     hipLaunchKernelGGL(dequantize_int4_scalar_kernel, dim3(grid_for(num_elements)), dim3(kBlock), 0, s,
                        static_cast<const uint8_t *>(packed_data), static_cast<const f16_t *>(scales), output,

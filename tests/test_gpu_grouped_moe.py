@@ -171,6 +171,68 @@ def test_moe_frozen_expert_layer_forward_backward(orc):
         assert max_rel_err(dxh[lo:hi], wdx) <= TOL
 
 
+def test_moe_frozen_expert_layer_full_size_config5(orc):
+    """BASELINE configs[4] at full size: 64 frozen SwiGLU experts (2048 -> 1408 -> 2048, int8 per-channel),
+    4096 tokens x top-6 = 24576 packed rows, forward (gate, up with the gating in its store, down) and the
+    backward chain to dX (src/caif_device_moe_frozen_expert.cpp:92-332).  The weights are quantised on the
+    device (its quantiser is checked against the oracle's elsewhere) and three experts' codes and scales are
+    brought back for the oracle: the first, a middle one and the last.  All experts are covered by the fused
+    launches giving the same bits as the reference's op-by-op sequence."""
+    rng = np.random.default_rng(640)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(640)
+    E, D, H, tokens, top_k = 64, 2048, 1408, 4096, 6
+    idx = rng.integers(0, E, (tokens, top_k)).astype(np.int32)
+    dmap, offsets, total = orc.moe_build_dispatch_map(idx, E)
+    assert total == tokens * top_k
+    sampled = (0, 29, 63)
+
+    def bank(N, K):
+        dws, ows = [], {}
+        for e in range(E):
+            w = torch.empty(K, N, device="cuda").normal_(0, 0.02, generator=gen)
+            q, s = T.quantize_int8(w, per_channel=True)              # [in, out] labelling: one scale per output
+            dws.append(T.FrozenWeight(q.reshape(-1), T.W_INT8, s, N, K, N))
+            if e in sampled:
+                ows[e] = orc.FrozenWeight(host(q).reshape(-1), orc.W_INT8, host(s), N, K, N, 128)
+        return ows, T.GroupedFrozenWeights(dws)
+
+    gate_o, gate_g = bank(H, D)
+    up_o, up_g = bank(H, D)
+    down_o, down_g = bank(D, H)
+    x = torch.empty(total, D, device="cuda").normal_(0, 1, generator=gen).to(torch.bfloat16)
+    g = torch.empty(total, D, device="cuda").normal_(0, 1e-2, generator=gen).to(torch.bfloat16)
+    off_d = dev(offsets)
+
+    # the layer as the host mirror runs it: gating folded into the up projection's store and into the store of
+    # the down projection's input gradient, the two input gradients summed in the second one's store
+    gate_out = T.qlinear_grouped_forward(x, off_d, gate_g, T.BF16, T.BF16)
+    up_out, hidden = T.qlinear_grouped_forward_swiglu(x, off_d, up_g, gate_out, T.BF16)
+    out = T.qlinear_grouped_forward(hidden, off_d, down_g, T.BF16, T.BF16)
+    grad_gate, grad_up = T.qlinear_grouped_backward_input_swiglu(g, off_d, down_g, gate_out, up_out, T.BF16)
+    gi_up = T.qlinear_grouped_backward_input(grad_up, off_d, up_g, T.BF16, T.BF16)
+    dx = T.qlinear_grouped_backward_input(grad_gate, off_d, gate_g, T.BF16, T.BF16, addend=gi_up)
+
+    # the reference's sequence, one op per launch: same bits on every row
+    up_ref = T.qlinear_grouped_forward(x, off_d, up_g, T.BF16, T.BF16)
+    hidden_ref = T.silu_multiply(gate_out, up_ref)
+    assert torch.equal(up_out, up_ref) and torch.equal(hidden, hidden_ref)
+    gh = T.qlinear_grouped_backward_input(g, off_d, down_g, T.BF16, T.BF16)
+    gg_ref, gu_ref = T.swiglu_backward(gate_out, up_ref, gh)
+    assert torch.equal(grad_gate, gg_ref) and torch.equal(grad_up, gu_ref)
+    gi_gate = T.qlinear_grouped_backward_input(gg_ref, off_d, gate_g, T.BF16, T.BF16)
+    assert torch.equal(dx, T.add(gi_up, gi_gate))
+
+    for e in sampled:
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        assert hi - lo >= 256, (e, hi - lo)
+        want, cache = orc.moe_frozen_expert_forward(host(x[lo:hi]), gate_o[e], up_o[e], down_o[e], 2, 2)
+        assert max_rel_err(host(hidden[lo:hi]), cache["hidden"]) <= TOL, e
+        assert max_rel_err(host(out[lo:hi]), want) <= TOL, e
+        wdx = orc.moe_frozen_expert_backward(host(g[lo:hi]), cache, gate_o[e], up_o[e], down_o[e], 2, 2)
+        assert max_rel_err(host(dx[lo:hi]), wdx) <= TOL, e
+
+
 def test_elementwise_ops_match_oracle(orc):
     rng = np.random.default_rng(4)
     n = 8 * 1000 + 5                                                 # vector body + scalar tail

@@ -26,7 +26,7 @@ def test_int8_per_tensor_bit_exact(orc, n):
     assert np.array_equal(host(d).view(np.uint32), orc.dequantize_int8_per_tensor(qo, so).view(np.uint32))
 
 
-@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (32, 64), (257, 129), (1024, 1408), (4096, 4096)])
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (32, 64), (37, 64), (70, 12), (257, 129), (1024, 1408), (4096, 4096)])
 def test_int8_per_channel_bit_exact(orc, shape):
     rng = np.random.default_rng(shape[0] * 7 + shape[1])
     x = _inputs(rng, shape[0] * shape[1]).reshape(shape)
@@ -38,6 +38,24 @@ def test_int8_per_channel_bit_exact(orc, shape):
     assert np.array_equal(host(q), qo)
     d = T.dequantize_int8(q, s, per_channel=True)
     assert np.array_equal(host(d).view(np.uint32), orc.dequantize_int8_per_channel(qo, so).view(np.uint32))
+
+
+def test_quantisers_on_buffers_that_are_not_16_byte_aligned(orc):
+    # views one element into a buffer: the kernels fall back from 16-byte to element accesses, same bits
+    rng = np.random.default_rng(5)
+    n, rows, cols = 4099, 37, 64
+    x = _inputs(rng, n)
+    buf = dev(np.concatenate([[0.0], x]).astype(np.float32))
+    q, s = T.quantize_int8(buf[1:], per_channel=False)
+    qo, so = orc.quantize_int8_per_tensor(x)
+    assert np.array_equal(host(s).view(np.uint32), so.view(np.uint32)) and np.array_equal(host(q), qo)
+    m = x[: rows * cols].reshape(rows, cols)
+    q, s = T.quantize_int8(buf[1 : 1 + rows * cols].view(rows, cols), per_channel=True)
+    qo, so = orc.quantize_int8_per_channel(m)
+    assert np.array_equal(host(s).view(np.uint32), so.view(np.uint32)) and np.array_equal(host(q), qo)
+    p, s = T.quantize_int4_per_group(buf[1 : 1 + 4096], 128)
+    po, so = orc.quantize_to_int4(x[:4096], 128)
+    assert np.array_equal(f16_bits(s), so) and np.array_equal(host(p), po)
 
 
 @pytest.mark.parametrize("n,group", [(4, 4), (5, 2), (512, 128), (128 * 37 + 77, 128), (1000, 24), (4096, 32),
