@@ -110,7 +110,13 @@ size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtyp
   a.compute_dtype = compute_dtype;
   a.w.kind = w_kind;
   const size_t f32_bytes = mfma_f32_workspace_bytes(a, backward != 0);
-  const size_t bytes = mfma_workspace_bytes(a, backward != 0);
+  size_t bytes = mfma_workspace_bytes(a, backward != 0);
+  if (!backward) {
+    // up to 32 rows go through the 16-row decode kernel, 16 rows at a time
+    if (a.M > 16 && a.M <= 32) a.M = 16;
+    const size_t decode_bytes = mblock_workspace_bytes(a);
+    if (decode_bytes > bytes) bytes = decode_bytes;
+  }
   return f32_bytes > bytes ? f32_bytes : bytes;
 }
 

@@ -68,6 +68,10 @@ struct MbArgs {
   int V;                 // residue classes the rows are split into (1 unless period > 0)
   int blocks_per_class;  // gridDim.x = blocks_per_class * V
   int scale_step;        // int8 scale vector: 1024 mod period (staging stride of the workgroup)
+  // K beyond one workgroup's reach: blockIdx.y takes the k range [y * slice_groups * 128, ...) and writes its
+  // share of the sums as fp32 to partial + y * M * N; a second launch adds the shares in a fixed order
+  int slice_groups;      // 128-k groups per slice (= groups when there is one slice)
+  float *partial;        // null with one slice
 };
 
 // 8 consecutive activations as compute-dtype values
@@ -160,6 +164,9 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
   const int nrb = i_hi > i_lo ? static_cast<int>((i_hi - i_lo + 15) / 16) : 0;
   if (nrb == 0) return;           // the whole workgroup; nothing has been started yet
   const int g0 = wave * GPW;
+  const int kbase = blockIdx.y * a.slice_groups * 128;          // first k of this workgroup's slice
+  const int groups = a.groups - blockIdx.y * a.slice_groups < a.slice_groups ? a.groups - blockIdx.y * a.slice_groups
+                                                                               : a.slice_groups;
   const f16_t *s16 = static_cast<const f16_t *>(a.scales);
   const float *s32 = static_cast<const float *>(a.scales);
 
@@ -168,10 +175,10 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
   auto issue = [&](int d, int rb) {
     int64_t i = i_lo + static_cast<int64_t>(rb) * 16 + j;
     if (i >= i_hi) i = i_hi - 1;                                   // masked lanes: their columns of the tile are never stored
-    const int64_t f0 = rb < nrb ? (cls + a.V * i) * a.K : 0;       // (wave uniform) past the end: the first weight row
+    const int64_t f0 = (rb < nrb ? (cls + a.V * i) * a.K : 0) + kbase;       // (wave uniform) past the end: the first weight row
 #pragma unroll
     for (int g = 0; g < GPW; ++g) {
-      const int gg = g0 + g < a.groups ? g0 + g : a.groups - 1;   // waves without a k range compute on zero activations
+      const int gg = g0 + g < groups ? g0 + g : groups - 1;   // waves without a k range compute on zero activations
       const int64_t f = f0 + gg * 128;
       if constexpr (kInt4) {
         w[d][g] = *reinterpret_cast<const u32x4_t *>(a.wq + (f >> 1) + q * 16);
@@ -187,10 +194,10 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
   // runs while the weights are still on their way from HBM.
   vec_t xa[GPW][4];
   {
-    const XT *xg = static_cast<const XT *>(a.x) + static_cast<int64_t>(j < a.M ? j : a.M - 1) * a.K;
+    const XT *xg = static_cast<const XT *>(a.x) + static_cast<int64_t>(j < a.M ? j : a.M - 1) * a.K + kbase;
 #pragma unroll
     for (int g = 0; g < GPW; ++g) {
-      const int gg = g0 + g < a.groups ? g0 + g : a.groups - 1;
+      const int gg = g0 + g < groups ? g0 + g : groups - 1;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const int k = kInt4 ? gg * 128 + q * 32 + 8 * t : gg * 128 + (t >> 1) * 64 + q * 16 + 8 * (t & 1);
@@ -203,7 +210,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
   float sv[4] = {1.0f, 1.0f, 1.0f, 1.0f};     // without a scale vector the staged scales are 1
   if constexpr (!kInt4) {
     if (a.period > 0) {
-      int idx = static_cast<int>((static_cast<int64_t>(cls) * a.K + threadIdx.x) % a.period);
+      int idx = static_cast<int>((static_cast<int64_t>(cls) * a.K + kbase + threadIdx.x) % a.period);
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         sv[t] = s32[idx];
@@ -223,7 +230,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
     for (int i = 0; i < 8; ++i) zero[i] = from_f32<CT>(0.0f);
 #pragma unroll
     for (int g = 0; g < GPW; ++g) {
-      const bool live = g0 + g < a.groups && j < a.M;
+      const bool live = g0 + g < groups && j < a.M;
 #pragma unroll
       for (int t = 0; t < 4; ++t) xa[g][t] = live ? xa[g][t] : zero;
     }
@@ -232,7 +239,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const int k = threadIdx.x + t * kMbThreads;
-      if (k < a.K) svec[k] = sv[t];
+      if (k < groups * 128) svec[k] = sv[t];
     }
   }
 
@@ -275,7 +282,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
     // four consecutive x' values: quad c (0..3) of step t
     auto xprime4 = [&](int t, int c, float (&v)[4]) {
       const int g = t >> 1;
-      const int gg = g0 + g < a.groups ? g0 + g : a.groups - 1;
+      const int gg = g0 + g < groups ? g0 + g : groups - 1;
       const vec_t xv = xa[g][2 * (t & 1) + (c >> 1)];
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] = to_f32<CT>(xv[4 * (c & 1) + i]);
@@ -417,10 +424,13 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
     // flush: Y[m][cls + V*i] for the rows of this segment
     const int64_t i_seg = i_lo + static_cast<int64_t>(seg0) * 16;
     const int seg_rows = static_cast<int>(i_hi - i_seg < kSegRows ? i_hi - i_seg : kSegRows);
+    float *part = a.partial ? a.partial + static_cast<int64_t>(blockIdx.y) * a.M * a.N : nullptr;
     for (int idx = threadIdx.x; idx < a.M * seg_rows; idx += kMbThreads) {
       const int m = idx / seg_rows;
       const int r = idx - m * seg_rows;
-      store_out(a.y, a.y_dtype, static_cast<int64_t>(m) * a.N + cls + a.V * (i_seg + r), ybuf[m * kSegRows + r]);
+      const int64_t o = static_cast<int64_t>(m) * a.N + cls + a.V * (i_seg + r);
+      if (part) part[o] = ybuf[m * kSegRows + r];
+      else store_out(a.y, a.y_dtype, o, ybuf[m * kSegRows + r]);
     }
   }
 }
@@ -438,10 +448,11 @@ int64_t gcd64(int64_t x, int64_t y)
 template <typename CT, typename XT, bool kInt4>
 int launch_gpw(const MbArgs &m, size_t lds, hipStream_t s)
 {
-  const unsigned grid = static_cast<unsigned>(m.blocks_per_class * m.V);
-  const int gpw = (m.groups + kMbWaves - 1) / kMbWaves;
-  if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 1>), dim3(grid), dim3(kMbThreads), lds, s, m);
-  else if (gpw <= 2) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 2>), dim3(grid), dim3(kMbThreads), lds, s, m);
+  const dim3 grid(static_cast<unsigned>(m.blocks_per_class * m.V),
+                  static_cast<unsigned>((m.groups + m.slice_groups - 1) / m.slice_groups));
+  const int gpw = (m.slice_groups + kMbWaves - 1) / kMbWaves;
+  if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 1>), grid, dim3(kMbThreads), lds, s, m);
+  else if (gpw <= 2) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 2>), grid, dim3(kMbThreads), lds, s, m);
   else return CAIFX_ERR_UNSUPPORTED;
   return launch_status();
 }
@@ -469,12 +480,27 @@ int compute_units()
 
 }  // namespace
 
+constexpr int64_t kMbSliceK = kMbWaves * 2 * 128;      // reduction length one workgroup covers
+
+size_t mblock_workspace_bytes(const GemmArgs &g)
+{
+  if (g.offsets || g.M < 1 || g.M > 16 || g.compute_dtype == CAIFX_F32 || g.K <= kMbSliceK || g.K % 128 != 0 ||
+      g.K > 64 * kMbSliceK)
+    return 0;
+  const int64_t slices = (g.K + kMbSliceK - 1) / kMbSliceK;
+  return static_cast<size_t>(slices) * static_cast<size_t>(g.M) * static_cast<size_t>(g.N) * sizeof(float);
+}
+
 int mblock_forward(const GemmArgs &g, hipStream_t s)
 {
   if (g.offsets || g.M < 1 || g.M > 16 || g.compute_dtype == CAIFX_F32) return CAIFX_ERR_UNSUPPORTED;
-  if (g.N < 16 || g.N > (int64_t{1} << 30) || g.K % 128 != 0 || g.K > kMbWaves * 2 * 128) return CAIFX_ERR_UNSUPPORTED;
+  if (g.N < 16 || g.N > (int64_t{1} << 30) || g.K % 128 != 0 || g.K > 64 * kMbSliceK) return CAIFX_ERR_UNSUPPORTED;
   if (!aligned_to(g.w.q, 16) || !aligned_to(g.x, 16)) return CAIFX_ERR_UNSUPPORTED;
   const bool int4 = g.w.kind == CAIFX_W_INT4_GROUP;
+  // a reduction longer than one workgroup's reach is cut into slices whose sums meet in the caller's workspace
+  const int64_t slices = (g.K + kMbSliceK - 1) / kMbSliceK;
+  if (slices > 1 && (!g.workspace || g.workspace_bytes < mblock_workspace_bytes(g) || !aligned_to(g.workspace, 4)))
+    return CAIFX_ERR_UNSUPPORTED;
 
   MbArgs m{};
   m.wq = static_cast<const uint8_t *>(g.w.q);
@@ -486,6 +512,8 @@ int mblock_forward(const GemmArgs &g, hipStream_t s)
   m.N = g.N;
   m.K = g.K;
   m.groups = static_cast<int>(g.K / 128);
+  m.slice_groups = slices > 1 ? static_cast<int>(kMbSliceK / 128) : m.groups;
+  m.partial = slices > 1 ? static_cast<float *>(g.workspace) : nullptr;
   m.V = 1;
   size_t lds = ((int4 ? 4 : 2) * kPartialFloats + 16 * kSegRows) * sizeof(float);      // RBB buffers of partial tiles + output staging
   if (int4) {
@@ -501,15 +529,19 @@ int mblock_forward(const GemmArgs &g, hipStream_t s)
     m.scale_step = static_cast<int>(kMbThreads % P);
     m.V = static_cast<int>(V);
   }
-  if (!int4) lds += static_cast<size_t>(g.K) * sizeof(float);      // staged scales (ones without a scale vector)
-  int target = compute_units();
+  if (!int4) lds += static_cast<size_t>(m.slice_groups) * 128 * sizeof(float);      // staged scales (ones without a scale vector)
+  // one workgroup per compute unit over all slices: the prologue (the slice of X as operands, for int8 its digit
+  // planes) is paid per workgroup, so each should own as many rows as the chip allows
+  int target = static_cast<int>((compute_units() + slices - 1) / slices);
   const int64_t nrb_class = ((g.N + m.V - 1) / m.V + 15) / 16;
   int64_t bpc = target / m.V;
   if (bpc < 1) bpc = 1;
   if (bpc > nrb_class) bpc = nrb_class;        // at least 16 rows per workgroup
   m.blocks_per_class = static_cast<int>(bpc);
-  if (g.compute_dtype == CAIFX_BF16) return launch_xt<bf16_t>(m, g.x_dtype, int4, lds, s);
-  return launch_xt<f16_t>(m, g.x_dtype, int4, lds, s);
+  const int st = g.compute_dtype == CAIFX_BF16 ? launch_xt<bf16_t>(m, g.x_dtype, int4, lds, s)
+                                                : launch_xt<f16_t>(m, g.x_dtype, int4, lds, s);
+  if (st != CAIFX_OK || slices == 1) return st;
+  return splitk_reduce(m.partial, static_cast<int>(slices), g.M * g.N, g.y, g.y_dtype, nullptr, s);
 }
 
 }  // namespace caifx

@@ -49,6 +49,8 @@ int rowlin_forward(const GemmArgs &a, hipStream_t s);
 // M <= 16 decode path on the matrix cores: activation rows are the A operand, so the cost per
 // weight byte does not grow with M.
 int mblock_forward(const GemmArgs &a, hipStream_t s);
+// Workspace of the above when the reduction is longer than one workgroup covers (K > 4096), else 0.
+size_t mblock_workspace_bytes(const GemmArgs &a);
 
 // Large-M MFMA path (compute bound), forward and input gradient, plain and grouped.
 int mfma_forward(const GemmArgs &a, hipStream_t s);

@@ -55,6 +55,27 @@ def test_decode_full_width_m1(orc, kind):
     _check(orc, np.random.default_rng(17), 1, 14336, 4096, kind, cd=2, xd=2)
 
 
+@pytest.mark.parametrize("kind", ["int4", "int8pc", "int8pt"])
+@pytest.mark.parametrize("N,K,M", [(4096, 14336, 1), (4096, 14336, 16), (1024, 8192, 4), (528, 11008, 9), (640, 4224, 24)])
+def test_reductions_longer_than_one_workgroup_covers(orc, kind, N, K, M):
+    # the FFN down projection (N = 4096, K = 14336) and other K > 4096: the 16-row decode kernel cuts the
+    # reduction into slices of 4096 (the last one shorter) whose sums meet in the workspace
+    rng = np.random.default_rng(N + K + M)
+    _check(orc, rng, M, N, K, kind, cd=2, xd=2)
+
+
+def test_long_reduction_without_a_workspace_takes_the_fallback(orc):
+    rng = np.random.default_rng(8)
+    N, K, M = 256, 8192, 5
+    ow, dw = make_weight(orc, rng, N, K, "int8pc")
+    xt = dev_as(rng.normal(0, 1, (M, K)), 2)
+    want = orc.frozen_linear_forward(host(xt), ow, 2)
+    import torch
+    none = torch.empty(0, dtype=torch.uint8, device="cuda")
+    y = host(T.qlinear_forward(xt, dw, 2, 0, workspace=none))
+    assert max_rel_err(y, want) <= TOL_16
+
+
 @pytest.mark.parametrize("cd,xd", [(2, 0), (2, 1), (1, 1), (1, 2), (1, 0)])
 @pytest.mark.parametrize("kind", ["int4", "int8pc"])
 def test_dtype_mixes(orc, kind, cd, xd):
