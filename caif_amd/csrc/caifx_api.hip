@@ -146,11 +146,19 @@ static int forward_impl(int64_t M, int64_t N, int64_t K, const void *x, int x_dt
   // one or two rows: stream each weight row linearly and reduce per row; from three rows on the
   // matrix-core tiling (cost independent of M) is faster; both fall through when a shape does not fit
   st = CAIFX_ERR_UNSUPPORTED;
-  // fp32 compute: from two rows on the fp32 matrix-core kernel (40-43 us at K = N = 4096 whatever M <= 32); the
-  // VALU decode kernel below takes 40-46 us for one row, 49-57 us for two and 66-71 us for four
-  if (compute_dtype == CAIFX_F32 && M > 1) {
-    st = mfma_f32_forward(a, s);
-    if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, y, y_dtype, M * N, stream);
+  // fp32 compute.  int8 storage with up to 16 rows: the 16-row decode kernel on the integer matrix core (digit
+  // planes of the fp32 activations); otherwise from two rows on the fp32 matrix-core kernel (40-43 us at
+  // K = N = 4096 whatever M <= 32); the VALU decode kernel below takes 40-46 us for one row
+  if (compute_dtype == CAIFX_F32) {
+    if (M <= 16 && w_kind == CAIFX_W_INT8) {
+      st = mblock_forward(a, s);
+      if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, y, y_dtype, M * N, stream);
+    }
+    if (M > 1) {
+      st = mfma_f32_forward(a, s);
+      if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, y, y_dtype, M * N, stream);
+    }
+    st = CAIFX_ERR_UNSUPPORTED;
   }
   if (M <= 2) st = rowlin_forward(a, s);
   if (st == CAIFX_ERR_UNSUPPORTED && M <= 16) {

@@ -136,9 +136,13 @@ constexpr int kSegRows = kSegBlocks * 16;
 // first bytes of the weight) and no global store happens between them (results are staged in LDS
 // and written once per kSegRows rows).  A wait for one block of the ring then leaves the younger
 // block in flight instead of draining the queue.
-template <typename CT, typename XT, bool kInt4, int GPW>
+// kF32 (int8 only): fp32 compute type.  The activations are not rounded to a 16-bit type: the digit planes are cut
+// from x * scale in fp32, read from memory in both passes over them instead of being kept in registers (CT then
+// only names a vector type nothing is stored in).
+template <typename CT, typename XT, bool kInt4, int GPW, bool kF32 = false>
 __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
 {
+  static_assert(!(kF32 && kInt4), "the fp32 compute type is for int8 storage");
   typedef typename Mfma16<CT>::vec_t vec_t;
   constexpr int LPG = kInt4 ? 1 : 2;           // 16-byte loads per lane per 128-k group
   constexpr int LPR = GPW * LPG;               // ... per block of 16 weight rows
@@ -193,8 +197,8 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
   // L2 and are needed first; then the first weight blocks.  Loads return in order, so the prologue
   // runs while the weights are still on their way from HBM.
   vec_t xa[GPW][4];
-  {
-    const XT *xg = static_cast<const XT *>(a.x) + static_cast<int64_t>(j < a.M ? j : a.M - 1) * a.K + kbase;
+  const XT *xg = static_cast<const XT *>(a.x) + static_cast<int64_t>(j < a.M ? j : a.M - 1) * a.K + kbase;
+  if constexpr (!kF32) {
 #pragma unroll
     for (int g = 0; g < GPW; ++g) {
       const int gg = g0 + g < groups ? g0 + g : groups - 1;
@@ -224,7 +228,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
 #pragma unroll
   for (int d = 0; d < D; ++d) issue(d, d);
 
-  {
+  if constexpr (!kF32) {
     vec_t zero;
 #pragma unroll
     for (int i = 0; i < 8; ++i) zero[i] = from_f32<CT>(0.0f);
@@ -283,9 +287,24 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
     auto xprime4 = [&](int t, int c, float (&v)[4]) {
       const int g = t >> 1;
       const int gg = g0 + g < groups ? g0 + g : groups - 1;
-      const vec_t xv = xa[g][2 * (t & 1) + (c >> 1)];
+      if constexpr (kF32) {
+        const bool live = g0 + g < groups && j < a.M;
+        const XT *px = xg + gg * 128 + (t & 1) * 64 + q * 16 + 4 * c;
+        if constexpr (sizeof(XT) == 4) {
+          const floatx4_t xv = *reinterpret_cast<const floatx4_t *>(px);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = to_f32<CT>(xv[4 * (c & 1) + i]);
+          for (int i = 0; i < 4; ++i) v[i] = live ? xv[i] : 0.0f;
+        } else {
+          const u32x2_t raw = *reinterpret_cast<const u32x2_t *>(px);
+          const XT *h = reinterpret_cast<const XT *>(&raw);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] = live ? to_f32<XT>(h[i]) : 0.0f;
+        }
+      } else {
+        const vec_t xv = xa[g][2 * (t & 1) + (c >> 1)];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = to_f32<CT>(xv[4 * (c & 1) + i]);
+      }
       const floatx4_t sc4 = *reinterpret_cast<const floatx4_t *>(svec + gg * 128 + (t & 1) * 64 + q * 16 + 4 * c);
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] *= sc4[i];
@@ -457,6 +476,18 @@ int launch_gpw(const MbArgs &m, size_t lds, hipStream_t s)
   return launch_status();
 }
 
+template <typename XT>
+int launch_f32(const MbArgs &m, size_t lds, hipStream_t s)
+{
+  const dim3 grid(static_cast<unsigned>(m.blocks_per_class * m.V),
+                  static_cast<unsigned>((m.groups + m.slice_groups - 1) / m.slice_groups));
+  const int gpw = (m.slice_groups + kMbWaves - 1) / kMbWaves;
+  if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<bf16_t, XT, false, 1, true>), grid, dim3(kMbThreads), lds, s, m);
+  else if (gpw <= 2) hipLaunchKernelGGL((mblock_kernel<bf16_t, XT, false, 2, true>), grid, dim3(kMbThreads), lds, s, m);
+  else return CAIFX_ERR_UNSUPPORTED;
+  return launch_status();
+}
+
 template <typename CT>
 int launch_xt(const MbArgs &m, int x_dtype, bool int4, size_t lds, hipStream_t s)
 {
@@ -484,19 +515,19 @@ constexpr int64_t kMbSliceK = kMbWaves * 2 * 128;      // reduction length one w
 
 size_t mblock_workspace_bytes(const GemmArgs &g)
 {
-  if (g.offsets || g.M < 1 || g.M > 16 || g.compute_dtype == CAIFX_F32 || g.K <= kMbSliceK || g.K % 128 != 0 ||
-      g.K > 64 * kMbSliceK)
-    return 0;
+  if (g.offsets || g.M < 1 || g.M > 16 || g.K <= kMbSliceK || g.K % 128 != 0 || g.K > 64 * kMbSliceK) return 0;
+  if (g.compute_dtype == CAIFX_F32 && g.w.kind == CAIFX_W_INT4_GROUP) return 0;
   const int64_t slices = (g.K + kMbSliceK - 1) / kMbSliceK;
   return static_cast<size_t>(slices) * static_cast<size_t>(g.M) * static_cast<size_t>(g.N) * sizeof(float);
 }
 
 int mblock_forward(const GemmArgs &g, hipStream_t s)
 {
-  if (g.offsets || g.M < 1 || g.M > 16 || g.compute_dtype == CAIFX_F32) return CAIFX_ERR_UNSUPPORTED;
+  if (g.offsets || g.M < 1 || g.M > 16) return CAIFX_ERR_UNSUPPORTED;
   if (g.N < 16 || g.N > (int64_t{1} << 30) || g.K % 128 != 0 || g.K > 64 * kMbSliceK) return CAIFX_ERR_UNSUPPORTED;
   if (!aligned_to(g.w.q, 16) || !aligned_to(g.x, 16)) return CAIFX_ERR_UNSUPPORTED;
   const bool int4 = g.w.kind == CAIFX_W_INT4_GROUP;
+  if (g.compute_dtype == CAIFX_F32 && int4) return CAIFX_ERR_UNSUPPORTED;
   // a reduction longer than one workgroup's reach is cut into slices whose sums meet in the caller's workspace
   const int64_t slices = (g.K + kMbSliceK - 1) / kMbSliceK;
   if (slices > 1 && (!g.workspace || g.workspace_bytes < mblock_workspace_bytes(g) || !aligned_to(g.workspace, 4)))
@@ -538,8 +569,13 @@ int mblock_forward(const GemmArgs &g, hipStream_t s)
   if (bpc < 1) bpc = 1;
   if (bpc > nrb_class) bpc = nrb_class;        // at least 16 rows per workgroup
   m.blocks_per_class = static_cast<int>(bpc);
-  const int st = g.compute_dtype == CAIFX_BF16 ? launch_xt<bf16_t>(m, g.x_dtype, int4, lds, s)
-                                                : launch_xt<f16_t>(m, g.x_dtype, int4, lds, s);
+  int st;
+  if (g.compute_dtype == CAIFX_F32)
+    st = g.x_dtype == CAIFX_F32 ? launch_f32<float>(m, lds, s)
+                                : (g.x_dtype == CAIFX_F16 ? launch_f32<f16_t>(m, lds, s) : launch_f32<bf16_t>(m, lds, s));
+  else
+    st = g.compute_dtype == CAIFX_BF16 ? launch_xt<bf16_t>(m, g.x_dtype, int4, lds, s)
+                                       : launch_xt<f16_t>(m, g.x_dtype, int4, lds, s);
   if (st != CAIFX_OK || slices == 1) return st;
   return splitk_reduce(m.partial, static_cast<int>(slices), g.M * g.N, g.y, g.y_dtype, nullptr, s);
 }
