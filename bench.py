@@ -544,12 +544,35 @@ def moe_rows(torch, T, dev, gen):
             routing[name].update({"GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                   "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
     routing_ms = sum(v["us"] for v in routing.values()) * 1e-3
+    # decode: 16 tokens x top-6 = 96 rows over the same 64 experts (one to four rows each, some none): the gate
+    # projection as one launch, memory bound on the touched experts' weights.  Two expert banks take turns so
+    # that the 370 MB of both do not stay in the Infinity Cache.
+    ids_d = torch.randint(0, E, (16 * top_k,), device=dev, generator=gen)
+    counts_d = torch.bincount(ids_d, minlength=E)
+    offs_d = torch.zeros(E + 1, dtype=torch.int32, device=dev)
+    offs_d[1:] = torch.cumsum(counts_d, 0).to(torch.int32)
+    xd = torch.empty(16 * top_k, D, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16)
+    yd = torch.empty(16 * top_k, H, device=dev)
+    banks = (gate, up)
+    turn = [0]
+
+    def decode_gate():
+        turn[0] ^= 1
+        T.qlinear_grouped_forward(xd, offs_d, banks[turn[0]], T.BF16, T.F32, out=yd, workspace=ws)
+
+    ms_d = timed(decode_gate, iters=20)
+    touched = int((counts_d > 0).sum())
+    dec_bytes = touched * (D * H + H * 4) + 16 * top_k * (D * 2 + H * 4)
+    decode = {"rows": 16 * top_k, "experts_touched": touched, "us": round(ms_d * 1e3, 2),
+              "GBps": round(dec_bytes / (ms_d * 1e-3) / 1e9, 1),
+              "frac_of_hbm_peak": round(dec_bytes / (ms_d * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     gemm_flops = 3 * 2.0 * rows * D * H
     return {"experts": E, "tokens": tokens, "top_k": top_k, "packed_rows": rows,
             "rows_per_expert_min_max": [int(counts.min()), int(counts.max())],
             "fwd_ms": round(ms_f, 4), "bwd_ms": round(ms_b, 4), "gating_in_gemm_store": {"fwd_ms": round(ms_f_fused, 4), "bwd_ms": round(ms_b_fused, 4)},
             "tokens_per_s_fwd_bwd": round(tokens / ((ms_f + ms_b) * 1e-3), 1),
             "routing": routing,
+            "decode_gate_projection_16_tokens": decode,
             "tokens_per_s_fwd_bwd_with_routing": round(tokens / ((ms_f + ms_b + routing_ms) * 1e-3), 1),
             "grouped_gemm_TFLOPs_fwd": round(gemm_flops / (ms_f * 1e-3) / 1e12, 1),
             "grouped_gemm_TFLOPs_bwd": round(gemm_flops / (ms_b * 1e-3) / 1e12, 1),

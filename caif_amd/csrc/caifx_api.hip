@@ -314,6 +314,11 @@ static int grouped(bool backward, int num_experts, const int32_t *offsets, int64
     st = backward ? mfma_f32_backward(a, s) : mfma_f32_forward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return st;
   }
+  if (!backward && !addend) {
+    // few rows per expert (MoE decode): memory bound on the touched experts' weights
+    st = mblock_grouped_forward(a, s);
+    if (st != CAIFX_ERR_UNSUPPORTED) return st;
+  }
   a.addend = addend;
   st = backward ? mfma_backward(a, s) : mfma_forward(a, s);
   if (st != CAIFX_ERR_UNSUPPORTED) return st;

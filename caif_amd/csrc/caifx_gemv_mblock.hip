@@ -139,8 +139,11 @@ constexpr int kSegRows = kSegBlocks * 16;
 // kF32 (int8 only): fp32 compute type.  The activations are not rounded to a 16-bit type: the digit planes are cut
 // from x * scale in fp32, read from memory in both passes over them instead of being kept in registers (CT then
 // only names a vector type nothing is stored in).
-template <typename CT, typename XT, bool kInt4, int GPW, bool kF32 = false>
-__global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
+// wq / scales: the weight; xrows / yrows: the first of the M <= 16 activation and result rows; slice: which part of
+// the reduction (see MbArgs).  Every thread of the workgroup makes the same calls (the body has barriers).
+template <typename CT, typename XT, bool kInt4, int GPW, bool kF32>
+__device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, const void *scales, const void *xrows,
+                                            void *yrows, int M, int slice)
 {
   static_assert(!(kF32 && kInt4), "the fp32 compute type is for int8 storage");
   typedef typename Mfma16<CT>::vec_t vec_t;
@@ -168,11 +171,11 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
   const int nrb = i_hi > i_lo ? static_cast<int>((i_hi - i_lo + 15) / 16) : 0;
   if (nrb == 0) return;           // the whole workgroup; nothing has been started yet
   const int g0 = wave * GPW;
-  const int kbase = blockIdx.y * a.slice_groups * 128;          // first k of this workgroup's slice
-  const int groups = a.groups - blockIdx.y * a.slice_groups < a.slice_groups ? a.groups - blockIdx.y * a.slice_groups
+  const int kbase = slice * a.slice_groups * 128;          // first k of this workgroup's slice
+  const int groups = a.groups - slice * a.slice_groups < a.slice_groups ? a.groups - slice * a.slice_groups
                                                                                : a.slice_groups;
-  const f16_t *s16 = static_cast<const f16_t *>(a.scales);
-  const float *s32 = static_cast<const float *>(a.scales);
+  const f16_t *s16 = static_cast<const f16_t *>(scales);
+  const float *s32 = static_cast<const float *>(scales);
 
   u32x4_t w[D][LPR];
   f16_t sc[D][GPW];
@@ -185,11 +188,11 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
       const int gg = g0 + g < groups ? g0 + g : groups - 1;   // waves without a k range compute on zero activations
       const int64_t f = f0 + gg * 128;
       if constexpr (kInt4) {
-        w[d][g] = *reinterpret_cast<const u32x4_t *>(a.wq + (f >> 1) + q * 16);
+        w[d][g] = *reinterpret_cast<const u32x4_t *>(wq + (f >> 1) + q * 16);
         sc[d][g] = s16[f >> a.group_shift];
       } else {
-        w[d][2 * g] = *reinterpret_cast<const u32x4_t *>(a.wq + f + q * 16);
-        w[d][2 * g + 1] = *reinterpret_cast<const u32x4_t *>(a.wq + f + 64 + q * 16);
+        w[d][2 * g] = *reinterpret_cast<const u32x4_t *>(wq + f + q * 16);
+        w[d][2 * g + 1] = *reinterpret_cast<const u32x4_t *>(wq + f + 64 + q * 16);
       }
     }
   };
@@ -197,7 +200,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
   // L2 and are needed first; then the first weight blocks.  Loads return in order, so the prologue
   // runs while the weights are still on their way from HBM.
   vec_t xa[GPW][4];
-  const XT *xg = static_cast<const XT *>(a.x) + static_cast<int64_t>(j < a.M ? j : a.M - 1) * a.K + kbase;
+  const XT *xg = static_cast<const XT *>(xrows) + static_cast<int64_t>(j < M ? j : M - 1) * a.K + kbase;
   if constexpr (!kF32) {
 #pragma unroll
     for (int g = 0; g < GPW; ++g) {
@@ -221,7 +224,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
         idx += a.scale_step;
         if (idx >= a.period) idx -= a.period;
       }
-    } else if (a.scales) {
+    } else if (scales) {
       s_one = s32[0];
     }
   }
@@ -234,7 +237,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
     for (int i = 0; i < 8; ++i) zero[i] = from_f32<CT>(0.0f);
 #pragma unroll
     for (int g = 0; g < GPW; ++g) {
-      const bool live = g0 + g < groups && j < a.M;
+      const bool live = g0 + g < groups && j < M;
 #pragma unroll
       for (int t = 0; t < 4; ++t) xa[g][t] = live ? xa[g][t] : zero;
     }
@@ -288,7 +291,7 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
       const int g = t >> 1;
       const int gg = g0 + g < groups ? g0 + g : groups - 1;
       if constexpr (kF32) {
-        const bool live = g0 + g < groups && j < a.M;
+        const bool live = g0 + g < groups && j < M;
         const XT *px = xg + gg * 128 + (t & 1) * 64 + q * 16 + 4 * c;
         if constexpr (sizeof(XT) == 4) {
           const floatx4_t xv = *reinterpret_cast<const floatx4_t *>(px);
@@ -443,14 +446,46 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
     // flush: Y[m][cls + V*i] for the rows of this segment
     const int64_t i_seg = i_lo + static_cast<int64_t>(seg0) * 16;
     const int seg_rows = static_cast<int>(i_hi - i_seg < kSegRows ? i_hi - i_seg : kSegRows);
-    float *part = a.partial ? a.partial + static_cast<int64_t>(blockIdx.y) * a.M * a.N : nullptr;
-    for (int idx = threadIdx.x; idx < a.M * seg_rows; idx += kMbThreads) {
+    float *part = a.partial ? a.partial + static_cast<int64_t>(slice) * M * a.N : nullptr;
+    for (int idx = threadIdx.x; idx < M * seg_rows; idx += kMbThreads) {
       const int m = idx / seg_rows;
       const int r = idx - m * seg_rows;
       const int64_t o = static_cast<int64_t>(m) * a.N + cls + a.V * (i_seg + r);
       if (part) part[o] = ybuf[m * kSegRows + r];
-      else store_out(a.y, a.y_dtype, o, ybuf[m * kSegRows + r]);
+      else store_out(yrows, a.y_dtype, o, ybuf[m * kSegRows + r]);
     }
+  }
+}
+
+template <typename CT, typename XT, bool kInt4, int GPW, bool kF32 = false>
+__global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
+{
+  mblock_body<CT, XT, kInt4, GPW, kF32>(a, a.wq, a.scales, a.x, a.y, a.M, blockIdx.y);
+}
+
+// Token-sorted expert segments with few rows each (MoE decode): blockIdx.y is the expert, whose weight is streamed
+// once per 16 rows of its segment; an expert without rows costs nothing.
+struct MbGroup {
+  const int32_t *offsets;
+  const void *const *wq_ptrs;
+  const void *const *scales_ptrs;
+  int64_t total_rows;
+};
+template <typename CT, typename XT, bool kInt4, int GPW>
+__global__ __launch_bounds__(kMbThreads) void mblock_grouped_kernel(MbArgs a, MbGroup g)
+{
+  const int e = blockIdx.y;
+  int lo, hi;
+  segment_rows(g.offsets, e, g.total_rows, lo, hi);
+  if (hi <= lo) return;
+  const uint8_t *wq = static_cast<const uint8_t *>(g.wq_ptrs[e]);
+  const void *scales = g.scales_ptrs ? g.scales_ptrs[e] : nullptr;
+  const size_t ybytes = a.y_dtype == CAIFX_F32 ? 4 : 2;
+  for (int r = lo; r < hi; r += 16) {
+    if (r > lo) __syncthreads();      // the pass before has read its staging buffers
+    mblock_body<CT, XT, kInt4, GPW, false>(a, wq, scales, static_cast<const XT *>(a.x) + static_cast<int64_t>(r) * a.K,
+                                           static_cast<char *>(a.y) + static_cast<int64_t>(r) * a.N * ybytes,
+                                           hi - r < 16 ? hi - r : 16, 0);
   }
 }
 
@@ -474,6 +509,27 @@ int launch_gpw(const MbArgs &m, size_t lds, hipStream_t s)
   else if (gpw <= 2) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 2>), grid, dim3(kMbThreads), lds, s, m);
   else return CAIFX_ERR_UNSUPPORTED;
   return launch_status();
+}
+
+template <typename CT, typename XT, bool kInt4>
+int launch_grouped_gpw(const MbArgs &m, const MbGroup &g, int experts, size_t lds, hipStream_t s)
+{
+  const dim3 grid(static_cast<unsigned>(m.blocks_per_class * m.V), static_cast<unsigned>(experts));
+  const int gpw = (m.groups + kMbWaves - 1) / kMbWaves;
+  if (gpw <= 1) hipLaunchKernelGGL((mblock_grouped_kernel<CT, XT, kInt4, 1>), grid, dim3(kMbThreads), lds, s, m, g);
+  else if (gpw <= 2) hipLaunchKernelGGL((mblock_grouped_kernel<CT, XT, kInt4, 2>), grid, dim3(kMbThreads), lds, s, m, g);
+  else return CAIFX_ERR_UNSUPPORTED;
+  return launch_status();
+}
+
+template <typename CT>
+int launch_grouped_xt(const MbArgs &m, const MbGroup &g, int experts, int x_dtype, bool int4, size_t lds, hipStream_t s)
+{
+  if (x_dtype == CAIFX_F32)
+    return int4 ? launch_grouped_gpw<CT, float, true>(m, g, experts, lds, s) : launch_grouped_gpw<CT, float, false>(m, g, experts, lds, s);
+  if (x_dtype == CAIFX_F16)
+    return int4 ? launch_grouped_gpw<CT, f16_t, true>(m, g, experts, lds, s) : launch_grouped_gpw<CT, f16_t, false>(m, g, experts, lds, s);
+  return int4 ? launch_grouped_gpw<CT, bf16_t, true>(m, g, experts, lds, s) : launch_grouped_gpw<CT, bf16_t, false>(m, g, experts, lds, s);
 }
 
 template <typename XT>
@@ -578,6 +634,51 @@ int mblock_forward(const GemmArgs &g, hipStream_t s)
                                        : launch_xt<f16_t>(m, g.x_dtype, int4, lds, s);
   if (st != CAIFX_OK || slices == 1) return st;
   return splitk_reduce(m.partial, static_cast<int>(slices), g.M * g.N, g.y, g.y_dtype, nullptr, s);
+}
+
+int mblock_grouped_forward(const GemmArgs &g, hipStream_t s)
+{
+  if (!g.offsets || !g.wq_ptrs || g.num_experts < 1 || g.num_experts > 65535 || g.compute_dtype == CAIFX_F32 || g.addend ||
+      g.epilogue != 0)
+    return CAIFX_ERR_UNSUPPORTED;
+  // worth it while a segment takes one or two passes of 16 rows; the tiled kernel streams an expert's weight
+  // once per 128 rows
+  if (g.M > 16 * static_cast<int64_t>(g.num_experts)) return CAIFX_ERR_UNSUPPORTED;
+  if (g.N < 16 || g.N > (int64_t{1} << 30) || g.K % 128 != 0 || g.K > kMbSliceK || !aligned_to(g.x, 16)) return CAIFX_ERR_UNSUPPORTED;
+  const bool int4 = g.w.kind == CAIFX_W_INT4_GROUP;
+  MbArgs m{};
+  m.x = g.x;
+  m.y = g.y;
+  m.M = 16;
+  m.y_dtype = g.y_dtype;
+  m.N = g.N;
+  m.K = g.K;
+  m.groups = static_cast<int>(g.K / 128);
+  m.slice_groups = m.groups;
+  m.V = 1;
+  size_t lds = ((int4 ? 4 : 2) * kPartialFloats + 16 * kSegRows) * sizeof(float);
+  if (int4) {
+    const int gs = g.w.group_size;
+    if (!g.scales_ptrs || gs < 128 || (gs & (gs - 1)) != 0) return CAIFX_ERR_UNSUPPORTED;
+    m.group_shift = __builtin_ctz(static_cast<unsigned>(gs));
+  } else if (g.scales_ptrs && g.w.scale_period > 1) {
+    const int64_t P = g.w.scale_period;
+    if (P > (int64_t{1} << 30)) return CAIFX_ERR_UNSUPPORTED;
+    const int64_t V = P / gcd64(g.K % P == 0 ? P : g.K % P, P);
+    if (V * 64 > g.N) return CAIFX_ERR_UNSUPPORTED;
+    m.period = static_cast<int>(P);
+    m.scale_step = static_cast<int>(kMbThreads % P);
+    m.V = static_cast<int>(V);
+  }
+  if (!int4) lds += static_cast<size_t>(g.K) * sizeof(float);
+  const int64_t nrb_class = ((g.N + m.V - 1) / m.V + 15) / 16;
+  int64_t bpc = 2 * static_cast<int64_t>(compute_units()) / (static_cast<int64_t>(g.num_experts) * m.V);
+  if (bpc < 1) bpc = 1;
+  if (bpc > nrb_class) bpc = nrb_class;
+  m.blocks_per_class = static_cast<int>(bpc);
+  MbGroup grp{g.offsets, g.wq_ptrs, g.scales_ptrs, g.M};
+  return g.compute_dtype == CAIFX_BF16 ? launch_grouped_xt<bf16_t>(m, grp, g.num_experts, g.x_dtype, int4, lds, s)
+                                       : launch_grouped_xt<f16_t>(m, grp, g.num_experts, g.x_dtype, int4, lds, s);
 }
 
 }  // namespace caifx

@@ -49,7 +49,10 @@ int rowlin_forward(const GemmArgs &a, hipStream_t s);
 // M <= 16 decode path on the matrix cores: activation rows are the A operand, so the cost per
 // weight byte does not grow with M.
 int mblock_forward(const GemmArgs &a, hipStream_t s);
-// Workspace of the above when the reduction is longer than one workgroup covers (K > 4096), else 0.
+// The same over token-sorted expert segments (forward), for launches with at most 16 rows per expert on average:
+// an expert's weight is streamed once per 16 rows of its segment.
+int mblock_grouped_forward(const GemmArgs &a, hipStream_t s);
+// Workspace of mblock_forward when the reduction is longer than one workgroup covers (K > 4096), else 0.
 size_t mblock_workspace_bytes(const GemmArgs &a);
 
 // Large-M MFMA path (compute bound), forward and input gradient, plain and grouped.

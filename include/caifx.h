@@ -208,7 +208,12 @@ CAIFX_API int caifx_qlinear_forward_static(int64_t M, int64_t N, int64_t K,
  * 0 <= lo <= hi <= total_rows per expert on the device: rows are lost, nothing
  * outside the buffers is touched).  wq_ptrs / scales_ptrs: device arrays of
  * E device pointers (one frozen linear per expert, each its own allocation as
- * in the reference); every expert shares N, K, kind, scale_period, group_size. */
+ * in the reference, 16-byte aligned); every expert shares N, K, kind, scale_period, group_size.
+ * Forward with total_rows <= 16 * num_experts (MoE decode: a few rows per expert), K <= 4096 and a 16-bit
+ * compute type runs the 16-row decode kernel over the segments: an expert's weight is streamed once per 16
+ * rows of its segment and an expert without rows costs nothing; the results carry that kernel's rounding
+ * (the weight is not rounded to the compute type, see caifx_qlinear_forward), a segment of 3..16 rows gets
+ * the bits of caifx_qlinear_forward on its rows. */
 CAIFX_API int caifx_qlinear_grouped_forward(int num_experts, const int32_t *offsets, int64_t total_rows,
                                   int64_t N, int64_t K,
                                   const void *x, int x_dtype, int compute_dtype,
