@@ -10,7 +10,7 @@ import os
 import subprocess
 
 F32, F16, BF16 = 0, 1, 2
-W_INT8, W_INT4_GROUP = 0, 1
+W_INT8, W_INT4_GROUP, W_F32, W_F16, W_BF16 = 0, 1, 2, 3, 4
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libcaifx.so")

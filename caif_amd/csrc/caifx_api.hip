@@ -28,6 +28,8 @@ void *static_scratch_on_current_device()
   return p;
 }
 
+bool float_kind(int w_kind) { return w_kind == CAIFX_W_F32 || w_kind == CAIFX_W_F16 || w_kind == CAIFX_W_BF16; }
+
 int validate_weight(int64_t N, int64_t K, int w_kind, const void *scales, int64_t scale_period, int group_size)
 {
   (void)N;
@@ -40,7 +42,7 @@ int validate_weight(int64_t N, int64_t K, int w_kind, const void *scales, int64_
       if (scale_period <= 0) return CAIFX_ERR_INVALID_ARGUMENT;
       if (!aligned_to(scales, 4)) return CAIFX_ERR_MISALIGNED;
     }
-  } else {
+  } else if (!float_kind(w_kind)) {
     return CAIFX_ERR_INVALID_ARGUMENT;
   }
   return CAIFX_OK;
@@ -70,7 +72,7 @@ GemmArgs make_args(int64_t M, int64_t N, int64_t K, const void *x, int x_dtype, 
   a.y_dtype = y_dtype;
   a.compute_dtype = compute_dtype;
   a.w.q = wq;
-  a.w.scales = scales;
+  a.w.scales = float_kind(w_kind) ? nullptr : scales;
   a.w.kind = w_kind;
   a.w.group_size = group_size;
   a.w.scale_period = (w_kind == CAIFX_W_INT8 && scales) ? scale_period : 1;
@@ -143,6 +145,11 @@ static int forward_impl(int64_t M, int64_t N, int64_t K, const void *x, int x_dt
   GemmArgs a = make_args(M, N, K, x, x_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, y,
                          y_dtype, workspace, workspace_bytes);
   hipStream_t s = as_stream(stream);
+  if (float_kind(w_kind)) {      // float storage: the fp32 matrix-core kernel, else the shape-agnostic one
+    st = mfma_f32_forward(a, s);
+    if (st == CAIFX_ERR_UNSUPPORTED) st = generic_forward(a, s);
+    return finish_add(st, addend, y, y_dtype, M * N, stream);
+  }
   // one or two rows: stream each weight row linearly and reduce per row; from three rows on the
   // matrix-core tiling (cost independent of M) is faster; both fall through when a shape does not fit
   st = CAIFX_ERR_UNSUPPORTED;
@@ -239,9 +246,10 @@ static int backward_impl(int64_t M, int64_t N, int64_t K, const void *dy, int dy
   GemmArgs a = make_args(M, N, K, dy, dy_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size,
                          dx, dx_dtype, workspace, workspace_bytes);
   hipStream_t s = as_stream(stream);
-  if (compute_dtype == CAIFX_F32) {
+  if (compute_dtype == CAIFX_F32 || float_kind(w_kind)) {
     st = mfma_f32_backward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, dx, dx_dtype, M * K, stream);
+    if (float_kind(w_kind)) return finish_add(generic_backward(a, s), addend, dx, dx_dtype, M * K, stream);
   }
   a.addend = addend;
   st = mfma_backward(a, s);
@@ -298,6 +306,8 @@ static int grouped(bool backward, int num_experts, const int32_t *offsets, int64
     if (group_size <= 0 || !scales_ptrs) return CAIFX_ERR_INVALID_ARGUMENT;
   } else if (w_kind == CAIFX_W_INT8) {
     if (scales_ptrs && scale_period <= 0) return CAIFX_ERR_INVALID_ARGUMENT;
+  } else if (float_kind(w_kind)) {
+    scales_ptrs = nullptr;
   } else {
     return CAIFX_ERR_INVALID_ARGUMENT;
   }
@@ -310,9 +320,13 @@ static int grouped(bool backward, int num_experts, const int32_t *offsets, int64
   a.num_experts = num_experts;
   if (addend && (addend == y || !aligned_to(addend, dtype_size(y_dtype)))) return CAIFX_ERR_INVALID_ARGUMENT;
   hipStream_t s = as_stream(stream);
-  if (compute_dtype == CAIFX_F32 && !addend) {
+  if ((compute_dtype == CAIFX_F32 || float_kind(w_kind)) && !addend) {
     st = backward ? mfma_f32_backward(a, s) : mfma_f32_forward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return st;
+  }
+  if (float_kind(w_kind)) {
+    if (addend) return CAIFX_ERR_UNSUPPORTED;
+    return backward ? generic_backward(a, s) : generic_forward(a, s);
   }
   if (!backward && !addend) {
     // few rows per expert (MoE decode): memory bound on the touched experts' weights
@@ -377,6 +391,8 @@ static int swiglu_grouped(bool backward, int num_experts, const int32_t *offsets
     if (group_size <= 0 || !scales_ptrs) return CAIFX_ERR_INVALID_ARGUMENT;
   } else if (w_kind == CAIFX_W_INT8) {
     if (scales_ptrs && scale_period <= 0) return CAIFX_ERR_INVALID_ARGUMENT;
+  } else if (float_kind(w_kind)) {
+    return CAIFX_ERR_UNSUPPORTED;        // the gated stores exist in the quantised kernels only
   } else {
     return CAIFX_ERR_INVALID_ARGUMENT;
   }

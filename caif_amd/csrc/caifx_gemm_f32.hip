@@ -42,6 +42,7 @@ struct F32Args {
   // part), and write fp32 partial tiles to d + part * M * C (d is then the caller's workspace)
   int parts;
   int part_steps;
+  int round_dt;          // float storage with a 16-bit compute type: operands are rounded to it (CAIFX_F32: not)
 };
 
 __device__ __forceinline__ void store_result(void *p, int dt, int64_t i, float v)
@@ -56,10 +57,16 @@ __device__ __forceinline__ void store_result(void *p, int dt, int64_t i, float v
 //    32 x 128 x 32: waves 1 x 4, 32 x 32 each
 //    32 x  32 x 128: every wave works on the whole tile and takes a quarter of each step's reduction
 // kVec: int8 with a scale vector (length a multiple of 4, 16-byte aligned: four scales per load)
-template <typename XT, bool kInt4, bool kVec, bool kBackward, int BM, int kBN, int kBK>
+// WT: void for quantised storage; float, f16_t or bf16_t for a weight stored undequantised (the float-storage cells of
+// the layer grid, src/caif_device_frozen_linear.cpp:301-318 and the .To(target) branch after them): its elements are
+// widened to fp32 and, like the activations, rounded to g.round_dt when that is a 16-bit type, so that the fp32
+// products and sums are those of a GEMM in that type with fp32 accumulation.
+template <typename XT, bool kInt4, bool kVec, bool kBackward, int BM, int kBN, int kBK, typename WT = void>
 __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
 {
   static_assert(kBN * kBK == 4096, "16 codes per thread and step");
+  constexpr bool kFloatW = !std::is_void<WT>::value;
+  constexpr int kWBytes = kFloatW ? static_cast<int>(sizeof(std::conditional_t<kFloatW, WT, char>)) : 1;
   constexpr bool kSplit = kBN == 32;       // the waves split the reduction instead of the tile
   constexpr int WM = BM == 128 ? 2 : 1;
   constexpr int WN = kSplit ? 1 : 4 / WM;
@@ -151,10 +158,17 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
       for (int e = 0; e < 4; ++e) areg[set][e] = to_f32<XT>(h[e]);
     }
   };
+  auto rounded = [&](float v) {
+    if constexpr (kFloatW) {
+      if (g.round_dt == CAIFX_BF16) return round_through<bf16_t>(v);
+      if (g.round_dt == CAIFX_F16) return round_through<f16_t>(v);
+    }
+    return v;
+  };
   auto store_a = [&](auto set_) {
     constexpr int set = decltype(set_)::value;
 #pragma unroll
-    for (int e = 0; e < EA; ++e) As[(a_col + e) * SA + a_row] = areg[set][e];
+    for (int e = 0; e < EA; ++e) As[(a_col + e) * SA + a_row] = rounded(areg[set][e]);
   };
 
   // ---- weights: 16 consecutive codes (along k) per thread and step
@@ -182,12 +196,19 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
   uint32_t sidx = vec_scales ? static_cast<uint32_t>(flat0 % g.period) : 0u;
   const float s_one = (!kInt4 && g.period == 1) ? s32[0] : 1.0f;
 
-  uint32_t wreg[2][kInt4 ? 2 : 4];
+  uint32_t wreg[2][kFloatW ? 4 * kWBytes : (kInt4 ? 2 : 4)];
   float sc[2][kInt4 ? 1 : 16];
   auto load_b = [&](auto set_, int s) {
     constexpr int set = decltype(set_)::value;
     const int64_t f = flat0 + static_cast<int64_t>(s) * flat_step;
-    if constexpr (kInt4) {
+    if constexpr (kFloatW) {
+#pragma unroll
+      for (int i = 0; i < kWBytes; ++i) {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(wq + f * kWBytes + 16 * i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) wreg[set][4 * i + e] = v[e];
+      }
+    } else if constexpr (kInt4) {
       const u32x2_t v = *reinterpret_cast<const u32x2_t *>(wq + (f >> 1));
       wreg[set][0] = v[0];
       wreg[set][1] = v[1];
@@ -217,7 +238,12 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
   auto store_b = [&](auto set_) {
     constexpr int set = decltype(set_)::value;
     float w[16];
-    if constexpr (kInt4) {
+    if constexpr (kFloatW) {
+      typedef std::conditional_t<kFloatW, WT, float> W_t;
+      const W_t *h = reinterpret_cast<const W_t *>(&wreg[set][0]);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) w[e] = rounded(to_f32<W_t>(h[e]));
+    } else if constexpr (kInt4) {
       float e0[8], e1[8];
       dequant_int4x8(wreg[set][0], sc[set][0], e0);
       dequant_int4x8(wreg[set][1], sc[set][0], e1);
@@ -331,7 +357,7 @@ __global__ __launch_bounds__(256) void qgemm_f32_kernel(F32Args g)
     }
 }
 
-template <typename XT, bool kInt4, bool kVec, bool kBackward>
+template <typename XT, bool kInt4, bool kVec, bool kBackward, typename WT = void>
 int launch_bm(const F32Args &f, hipStream_t s)
 {
   const int64_t C = kBackward ? f.K : f.N;
@@ -344,13 +370,13 @@ int launch_bm(const F32Args &f, hipStream_t s)
     const int64_t row_tiles = (f.M + (tall_tiles ? 127 : 31)) / (tall_tiles ? 128 : 32) + f.num_experts;
     if (row_tiles > 65535) return CAIFX_ERR_UNSUPPORTED;
     const dim3 grid(static_cast<unsigned>(col_tiles), static_cast<unsigned>(row_tiles));
-    if (tall_tiles) hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 128, 128, 32>), grid, dim3(256), 0, s, f);
-    else hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 128, 32>), grid, dim3(256), 0, s, f);
+    if (tall_tiles) hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 128, 128, 32, WT>), grid, dim3(256), 0, s, f);
+    else hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 128, 32, WT>), grid, dim3(256), 0, s, f);
     return launch_status();
   }
   // few rows: 32 x 32 tiles whose waves split the reduction (128-deep steps)
   if (f.M <= kSplitTileRows && R % 128 == 0) {
-    hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 32, 128>),
+    hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 32, 128, WT>),
                        dim3(static_cast<unsigned>((C + 31) / 32), static_cast<unsigned>((f.M + 31) / 32), static_cast<unsigned>(f.parts)),
                        dim3(256), 0, s, f);
     return launch_status();
@@ -359,20 +385,23 @@ int launch_bm(const F32Args &f, hipStream_t s)
   // put four times as many workgroups on the chip for the same weight traffic through L2
   const int64_t tall = (f.M + 127) / 128;
   if (tall * col_tiles >= 256 && tall <= 65535) {
-    hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 128, 128, 32>), dim3(static_cast<unsigned>(col_tiles), static_cast<unsigned>(tall)),
+    hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 128, 128, 32, WT>), dim3(static_cast<unsigned>(col_tiles), static_cast<unsigned>(tall)),
                        dim3(256), 0, s, f);
     return launch_status();
   }
   const int64_t low = (f.M + 31) / 32;
   if (low > 65535) return CAIFX_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 128, 32>), dim3(static_cast<unsigned>(col_tiles), static_cast<unsigned>(low)),
+  hipLaunchKernelGGL((qgemm_f32_kernel<XT, kInt4, kVec, kBackward, 32, 128, 32, WT>), dim3(static_cast<unsigned>(col_tiles), static_cast<unsigned>(low)),
                      dim3(256), 0, s, f);
   return launch_status();
 }
 
 template <typename XT>
-int launch_kind(const F32Args &f, bool int4, bool backward, hipStream_t s)
+int launch_kind(const F32Args &f, int kind, bool int4, bool backward, hipStream_t s)
 {
+  if (kind == CAIFX_W_F32) return backward ? launch_bm<XT, false, false, true, float>(f, s) : launch_bm<XT, false, false, false, float>(f, s);
+  if (kind == CAIFX_W_F16) return backward ? launch_bm<XT, false, false, true, f16_t>(f, s) : launch_bm<XT, false, false, false, f16_t>(f, s);
+  if (kind == CAIFX_W_BF16) return backward ? launch_bm<XT, false, false, true, bf16_t>(f, s) : launch_bm<XT, false, false, false, bf16_t>(f, s);
   if (int4) return backward ? launch_bm<XT, true, false, true>(f, s) : launch_bm<XT, true, false, false>(f, s);
   if (f.period > 1) return backward ? launch_bm<XT, false, true, true>(f, s) : launch_bm<XT, false, true, false>(f, s);
   return backward ? launch_bm<XT, false, false, true>(f, s) : launch_bm<XT, false, false, false>(f, s);
@@ -408,7 +437,8 @@ F32Plan plan_f32(int64_t M, int64_t C, int64_t R, bool grouped)
 
 int run_f32(const GemmArgs &a, bool backward, hipStream_t s)
 {
-  if (a.compute_dtype != CAIFX_F32 || a.addend || a.epilogue) return CAIFX_ERR_UNSUPPORTED;
+  const bool float_w = a.w.kind == CAIFX_W_F32 || a.w.kind == CAIFX_W_F16 || a.w.kind == CAIFX_W_BF16;
+  if ((a.compute_dtype != CAIFX_F32 && !float_w) || a.addend || a.epilogue) return CAIFX_ERR_UNSUPPORTED;
   const bool grouped = a.offsets != nullptr;
   if (grouped && (a.num_experts < 1 || !a.wq_ptrs)) return CAIFX_ERR_UNSUPPORTED;
   const int64_t R = backward ? a.N : a.K;
@@ -449,9 +479,10 @@ int run_f32(const GemmArgs &a, bool backward, hipStream_t s)
       f.period = a.w.scale_period;
       f.step = static_cast<uint32_t>((backward ? static_cast<int64_t>(kStep) * a.K : kStep) % a.w.scale_period);
     }
-  } else {
+  } else if (!float_w) {
     return CAIFX_ERR_UNSUPPORTED;
   }
+  f.round_dt = float_w ? a.compute_dtype : CAIFX_F32;
   f.parts = 1;
   const int64_t cols = backward ? a.K : a.N;
   const F32Plan plan = plan_f32(a.M, cols, R, grouped);
@@ -463,9 +494,9 @@ int run_f32(const GemmArgs &a, bool backward, hipStream_t s)
     f.d_dtype = CAIFX_F32;
   }
   int st;
-  if (a.x_dtype == CAIFX_F32) st = launch_kind<float>(f, int4, backward, s);
-  else if (a.x_dtype == CAIFX_BF16) st = launch_kind<bf16_t>(f, int4, backward, s);
-  else if (a.x_dtype == CAIFX_F16) st = launch_kind<f16_t>(f, int4, backward, s);
+  if (a.x_dtype == CAIFX_F32) st = launch_kind<float>(f, a.w.kind, int4, backward, s);
+  else if (a.x_dtype == CAIFX_BF16) st = launch_kind<bf16_t>(f, a.w.kind, int4, backward, s);
+  else if (a.x_dtype == CAIFX_F16) st = launch_kind<f16_t>(f, a.w.kind, int4, backward, s);
   else return CAIFX_ERR_UNSUPPORTED;
   if (!shared || st != CAIFX_OK) return st;
   return splitk_reduce(static_cast<const float *>(a.workspace), plan.parts, a.M * cols, a.y, a.y_dtype, nullptr, s);
@@ -475,7 +506,8 @@ int run_f32(const GemmArgs &a, bool backward, hipStream_t s)
 
 size_t mfma_f32_workspace_bytes(const GemmArgs &a, bool backward)
 {
-  if (a.compute_dtype != CAIFX_F32) return 0;
+  const bool float_w = a.w.kind == CAIFX_W_F32 || a.w.kind == CAIFX_W_F16 || a.w.kind == CAIFX_W_BF16;
+  if (a.compute_dtype != CAIFX_F32 && !float_w) return 0;
   return plan_f32(a.M, backward ? a.K : a.N, backward ? a.N : a.K, a.offsets != nullptr).bytes;
 }
 

@@ -33,7 +33,13 @@ __device__ __forceinline__ float weight_rt(const QWeight &w, const void *wq, con
                                            int compute_dtype)
 {
   float v;
-  if (w.kind == CAIFX_W_INT4_GROUP) {
+  if (w.kind == CAIFX_W_F32) {
+    v = static_cast<const float *>(wq)[f];
+  } else if (w.kind == CAIFX_W_F16) {
+    v = to_f32(static_cast<const f16_t *>(wq)[f]);
+  } else if (w.kind == CAIFX_W_BF16) {
+    v = to_f32(static_cast<const bf16_t *>(wq)[f]);
+  } else if (w.kind == CAIFX_W_INT4_GROUP) {
     const uint32_t b = static_cast<const uint8_t *>(wq)[f >> 1];
     v = static_cast<float>(nibble_s4(b, static_cast<int>(f & 1))) *
         to_f32(static_cast<const f16_t *>(scales)[f / w.group_size]);

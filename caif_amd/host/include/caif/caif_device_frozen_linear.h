@@ -39,8 +39,10 @@ template<typename ComputeT=float,typename StorageT=int8_t>
 class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
                               public CAIF_DeviceFrozenLinearBase
 {
-  static_assert(std::is_same<StorageT,int8_t>::value||std::is_same<StorageT,caif_int4_packed_t>::value,
-                "CAIF_DeviceFrozenLinear: this build covers the int8 and int4 storage cells");
+  static_assert(std::is_same<StorageT,int8_t>::value||std::is_same<StorageT,caif_int4_packed_t>::value||
+                std::is_same<StorageT,float>::value||std::is_same<StorageT,caif_fp16_t>::value||
+                std::is_same<StorageT,caif_bf16_t>::value,
+                "CAIF_DeviceFrozenLinear: storage is int8, packed int4 or one of the three float types");
 
   public:
     typedef CAIF_DeviceLayerTyped<ComputeT,StorageT> Base_t;
@@ -187,6 +189,13 @@ class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
         CAIF_DeviceTensor fp32=CAIF_DeviceTensor::Uninitialized({OutputDim(),InputDim()},Stream());
         hipStream_t s=Stream().Handle();
         int st;
+        if(IsFloatStorage()==true)
+        {
+          // float storage: the weight itself, widened (src/caif_device_frozen_linear.cpp:780-790)
+          CAIF_DeviceTensor wide=_weight.To(Dtype_e::Float32);
+          wide.Reshape({OutputDim(),InputDim()});
+          return wide;
+        }
         if(IsInt4()==true)
         {
           if(_scales.IsEmpty()==true){THROW_CAIFE("FrozenLinear: scales not loaded");}
@@ -282,12 +291,15 @@ class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
     {
       try
       {
-        if(_weight.IsEmpty()==true||_scales.IsEmpty()==true)
+        if(_weight.IsEmpty()==true||(IsFloatStorage()==false&&_scales.IsEmpty()==true))
         {
           THROW_CAIFE("FrozenLinear::ExportQuantized: weight and scales must be loaded (and resident on the device)");
         }
         tensors.emplace_back(prefix+"weight",&_weight);
-        tensors.emplace_back(prefix+"scales",&_scales);
+        if(IsFloatStorage()==false)
+        {
+          tensors.emplace_back(prefix+"scales",&_scales);
+        }
         metadata[prefix+"storage"]=CAIF_DataType(Base_t::StorageDtype()).Name();
         metadata[prefix+"group_size"]=std::to_string(_group_size);
         metadata[prefix+"int8_scheme"]=SchemeName(_int8_scheme);
@@ -304,7 +316,7 @@ class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
       {
         auto w=tensors.find(prefix+"weight");
         auto s=tensors.find(prefix+"scales");
-        if(w==tensors.end()||s==tensors.end())
+        if(w==tensors.end()||(s==tensors.end()&&IsFloatStorage()==false))
         {
           THROW_CAIFE("FrozenLinear::ImportQuantized: missing tensor "+prefix+(w==tensors.end()?"weight":"scales"));
         }
@@ -325,7 +337,7 @@ class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
         {
           THROW_CAIFE("FrozenLinear::ImportQuantized: group size does not match the layer");
         }
-        if(IsInt4()==false&&meta("int8_scheme")!=SchemeName(_int8_scheme))
+        if(IsInt4()==false&&IsFloatStorage()==false&&meta("int8_scheme")!=SchemeName(_int8_scheme))
         {
           THROW_CAIFE("FrozenLinear::ImportQuantized: int8 scheme does not match the layer");
         }
@@ -333,7 +345,10 @@ class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
         {
           THROW_CAIFE("FrozenLinear::ImportQuantized: weight shape must be [output_dim, input_dim]");
         }
-        LoadScalesFromTensor(std::move(s->second));
+        if(IsFloatStorage()==false)
+        {
+          LoadScalesFromTensor(std::move(s->second));
+        }
         LoadFromTensor(std::move(w->second));
         tensors.erase(prefix+"weight");
         tensors.erase(prefix+"scales");
@@ -341,7 +356,7 @@ class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
       CAIF_CATCH_BLOCK()
     }
     void ClearFP32Cache()override{}
-    bool NeedsScales()const override{return true;}
+    bool NeedsScales()const override{return IsFloatStorage()==false;}
     CAIF_Ops::QuantScheme_e Int8Scheme()const override{return _int8_scheme;}
     bool CacheFP32()const override{return _cache_fp32;}
     uint32_t InputDim()const override{return _input_dim;}
@@ -351,10 +366,16 @@ class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
     // Raw views for callers that batch several layers into one grouped launch.
     const void *WeightData()const{return _weight.DeviceDataRaw();}
     const void *ScalesData()const{return _scales.IsEmpty()?nullptr:_scales.DeviceDataRaw();}
-    int WeightKind()const{return IsInt4()?CAIFX_W_INT4_GROUP:CAIFX_W_INT8;}
+    int WeightKind()const
+    {
+      if(std::is_same<StorageT,float>::value){return CAIFX_W_F32;}
+      if(std::is_same<StorageT,caif_fp16_t>::value){return CAIFX_W_F16;}
+      if(std::is_same<StorageT,caif_bf16_t>::value){return CAIFX_W_BF16;}
+      return IsInt4()?CAIFX_W_INT4_GROUP:CAIFX_W_INT8;
+    }
     int64_t ScalePeriod()const
     {
-      return (IsInt4()==false&&_int8_scheme==CAIF_Ops::QuantScheme_e::PerChannel_e)?static_cast<int64_t>(OutputDim()):1;
+      return (IsInt4()==false&&IsFloatStorage()==false&&_int8_scheme==CAIF_Ops::QuantScheme_e::PerChannel_e)?static_cast<int64_t>(OutputDim()):1;
     }
 
     // --- CPU offload surface (src/caif_device_frozen_linear.cpp:145-232) ---
@@ -414,11 +435,16 @@ class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
 
   private:
     static constexpr bool IsInt4(){return std::is_same<StorageT,caif_int4_packed_t>::value;}
+    static constexpr bool IsFloatStorage()
+    {
+      return std::is_same<StorageT,float>::value||std::is_same<StorageT,caif_fp16_t>::value||
+             std::is_same<StorageT,caif_bf16_t>::value;
+    }
     static const char *SchemeName(CAIF_Ops::QuantScheme_e s)
     {
       return s==CAIF_Ops::QuantScheme_e::PerChannel_e?"per_channel":"per_tensor";
     }
-    const void *ScalesPtr()const{return _scales.IsEmpty()?nullptr:_scales.DeviceDataRaw();}
+    const void *ScalesPtr()const{return (IsFloatStorage()||_scales.IsEmpty())?nullptr:_scales.DeviceDataRaw();}
     void RequireScales()const
     {
       if(IsInt4()==true&&_scales.IsEmpty()==true){THROW_CAIFE("FrozenLinear: scales not loaded");}

@@ -1,8 +1,8 @@
 // Runtime (storage dtype, compute dtype) -> template cell.  Signature of
 // CAIF_DeviceFrozenLinearFactory::Create (src/caif_device_frozen_linear_factory.cpp:46-54); callers
 // dynamic_cast the result to CAIF_DeviceFrozenLinearBase* to load weights and scales
-// (tests/test_device_frozen_linear.cpp:237-238).  The six quantised cells are built; the nine
-// float-storage cells of the reference's grid are rejected (they are not on the quantised path).
+// (tests/test_device_frozen_linear.cpp:237-238).  All fifteen cells of the reference's grid are built; the nine
+// float-storage ones run on the fp32 matrix-core kernel (they are not on the quantised fast paths).
 #pragma once
 
 #include <memory>
@@ -33,7 +33,19 @@ class CAIF_DeviceFrozenLinearFactory
         {
           return ByCompute<caif_int4_packed_t>(input_dim,output_dim,stream,group_size,cache_fp32,compute_dtype,int8_scheme);
         }
-        THROW_CAIFE("FrozenLinearFactory: only Int8 and Int4 storage are built (float storage cells are out of scope)");
+        if(storage_dtype==Dtype_e::Float32)
+        {
+          return ByCompute<float>(input_dim,output_dim,stream,group_size,cache_fp32,compute_dtype,int8_scheme);
+        }
+        if(storage_dtype==Dtype_e::Float16)
+        {
+          return ByCompute<caif_fp16_t>(input_dim,output_dim,stream,group_size,cache_fp32,compute_dtype,int8_scheme);
+        }
+        if(storage_dtype==Dtype_e::BFloat16)
+        {
+          return ByCompute<caif_bf16_t>(input_dim,output_dim,stream,group_size,cache_fp32,compute_dtype,int8_scheme);
+        }
+        THROW_CAIFE("FrozenLinearFactory: unsupported storage dtype");
       }
       CAIF_CATCH_BLOCK()
     }

@@ -7,7 +7,7 @@ points (src/caif_ops.cpp:504-680); argument meaning is the same.
 import torch
 
 from . import capi
-from .capi import F32, F16, BF16, W_INT8, W_INT4_GROUP
+from .capi import F32, F16, BF16, W_INT8, W_INT4_GROUP, W_F32, W_F16, W_BF16
 
 TORCH_DTYPE = {F32: torch.float32, F16: torch.float16, BF16: torch.bfloat16}
 CODE_OF = {v: k for k, v in TORCH_DTYPE.items()}

@@ -63,8 +63,14 @@ enum caifx_dtype { CAIFX_F32 = 0, CAIFX_F16 = 1, CAIFX_BF16 = 2 };
  *                      src/caif_cuda_kernels_quant.cu:561-574).  scales == NULL is the
  *                      "int8 without scales" branch, a plain widening cast (:373-375).
  *  CAIFX_W_INT4_GROUP: packed nibbles; W[n,k] = code * fp16 scales[(n*K+k) / group_size]
- *                      (src/caif_cuda_kernels_quant.cu:233-235). */
-enum caifx_weight_kind { CAIFX_W_INT8 = 0, CAIFX_W_INT4_GROUP = 1 };
+ *                      (src/caif_cuda_kernels_quant.cu:233-235).
+ *  CAIFX_W_F32 / CAIFX_W_F16 / CAIFX_W_BF16: the weight stored undequantised in that float type, W[n,k] =
+ *                      element n*K+k cast to the compute type (the float-storage cells of the layer grid:
+ *                      src/caif_device_frozen_linear.cpp:301-318 uses the buffer as it is when storage and
+ *                      compute types agree, otherwise Weight().To(target)); scales, scale_period and group_size
+ *                      are ignored.  These cells run on the fp32 matrix-core kernel (operands rounded to a
+ *                      16-bit compute type first, fp32 products and sums), not on the fast paths of the quantised kinds. */
+enum caifx_weight_kind { CAIFX_W_INT8 = 0, CAIFX_W_INT4_GROUP = 1, CAIFX_W_F32 = 2, CAIFX_W_F16 = 3, CAIFX_W_BF16 = 4 };
 
 CAIFX_API const char *caifx_status_string(int status);
 /* ABI version of this header: major*1000 + minor. */

@@ -43,7 +43,7 @@ ORC_API int orc_max_threads(void)
 /* dtype codes shared with include/caifx.h */
 enum { ORC_F32 = 0, ORC_F16 = 1, ORC_BF16 = 2 };
 /* weight kinds shared with include/caifx.h */
-enum { ORC_W_INT8 = 0, ORC_W_INT4_GROUP = 1 };
+enum { ORC_W_INT8 = 0, ORC_W_INT4_GROUP = 1, ORC_W_F32 = 2, ORC_W_F16 = 3, ORC_W_BF16 = 4 };
 
 /* include/caif/caif_cuda_kernels_constants.cuh:185-197 */
 static const float k_int8_max = 127.0f;
@@ -285,13 +285,23 @@ ORC_API void orc_dequantize_int4(const uint8_t *packed, const uint16_t *scales_f
  * rows=InputDim, cols=OutputDim (:356-361), i.e. scale index = f % N; that is
  * the `scale_period` here (1 for per-tensor).  scales == NULL reproduces the
  * int8-without-scales branch (:373-375), a plain widening cast.
+ * Float storage (ORC_W_F32 / F16 / BF16): the buffer as it is when storage and
+ * compute types agree (:301-318), otherwise its elements cast to the compute
+ * type (the tensor's .To(target): widen to fp32, round to nearest even).
  * w_out holds the compute-dtype values widened to fp32. */
 ORC_API void orc_frozen_weight_compute(const void *wq, int w_kind, const void *scales,
                                        int64_t N, int64_t K, int64_t scale_period, int group_size,
                                        int compute_dtype, float *w_out)
 {
   int64_t total = N * K;
-  if (w_kind == ORC_W_INT4_GROUP) {
+  if (w_kind == ORC_W_F32) {
+    memcpy(w_out, wq, (size_t)total * sizeof(float));
+  } else if (w_kind == ORC_W_F16 || w_kind == ORC_W_BF16) {
+    const uint16_t *h = (const uint16_t *)wq;
+#pragma omp parallel for schedule(static)
+    for (int64_t f = 0; f < total; ++f)
+      w_out[f] = w_kind == ORC_W_F16 ? orc_f16_to_f32(h[f]) : orc_bf16_to_f32(h[f]);
+  } else if (w_kind == ORC_W_INT4_GROUP) {
     orc_dequantize_int4((const uint8_t *)wq, (const uint16_t *)scales, w_out, total, group_size);
   } else {
     const int8_t *q = (const int8_t *)wq;

@@ -19,7 +19,7 @@ import subprocess
 import numpy as np
 
 F32, F16, BF16 = 0, 1, 2            # dtype codes (same as include/caifx.h)
-W_INT8, W_INT4_GROUP = 0, 1         # weight kinds (same as include/caifx.h)
+W_INT8, W_INT4_GROUP, W_F32, W_F16, W_BF16 = 0, 1, 2, 3, 4         # weight kinds (same as include/caifx.h)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libcaif_oracle.so")
@@ -219,7 +219,11 @@ def dequantize_int4(packed, scales_f16_bits, n, group_size):
 def frozen_weight_compute(wq, w_kind, scales, N, K, scale_period, group_size, compute_dtype):
     """W[N,K] in the compute dtype, as ConvertToComputeDtype materialises it
     (src/caif_device_frozen_linear.cpp:289-378)."""
-    if w_kind == W_INT4_GROUP:
+    if w_kind == W_F32:
+        wq, scales = _c(wq, np.float32), None
+    elif w_kind in (W_F16, W_BF16):           # the 16-bit patterns of the stored elements
+        wq, scales = _c(wq, np.uint16), None
+    elif w_kind == W_INT4_GROUP:
         wq = _c(wq, np.uint8)
         scales = _c(scales, np.uint16)
     else:

@@ -96,6 +96,36 @@ static void GpuTests()
     }
   }
   {
+    // Float storage: the nine remaining cells of the grid.  The weight is loaded as stored ([output_dim, input_dim],
+    // the layout tests/test_device_frozen_linear.cpp:996-1072 pins against a dense layer), no scales.
+    const Dtype_e storages[3]={Dtype_e::Float32,Dtype_e::Float16,Dtype_e::BFloat16};
+    for(int si=0;si<3;++si)
+    {
+      for(int ci=0;ci<3;++ci)
+      {
+        auto layer=CAIF_DeviceFrozenLinearFactory::Create(K,N,storages[si],stream,16,true,computes[ci]);
+        CAIF_DeviceFrozenLinearBase *base=dynamic_cast<CAIF_DeviceFrozenLinearBase*>(layer.get());
+        CAIF_DeviceTensor wt=Upload(w,{N,K},stream);
+        base->LoadFromTensor(storages[si]==Dtype_e::Float32?std::move(wt):wt.To(storages[si]));
+        const std::string tag=std::string("float storage ")+CAIF_DataType(storages[si]).Name()+" / "+CAIF_DataType(computes[ci]).Name();
+        Report(tag+": needs no scales",base->NeedsScales()==false);
+        CAIF_DeviceTensor in=Upload(x,{M,K},stream);
+        CAIF_DeviceTensor out=layer->Forward(in,infer);
+        const bool exact=storages[si]==Dtype_e::Float32&&computes[ci]==Dtype_e::Float32;
+        const float tol=exact?1e-5f:2e-2f;
+        Report(tag+": forward matches the dense product",out.Dtype()==Dtype_e::Float32&&out.Shape()==std::vector<uint32_t>({M,N})&&
+                                                         RelToMax(Download(out),ref)<=tol);
+        const std::vector<float> wd=Download(layer->FrozenTensorFP32(0));
+        Report(tag+": frozen tensor is the stored weight widened",RelToMax(wd,w)<=(storages[si]==Dtype_e::Float32?0.0f:1e-2f));
+        layer->Forward(in,train);
+        CAIF_DeviceTensor go=Upload(g,{M,N},stream);
+        CAIF_DeviceTensor dx=layer->Backward(go,train);
+        Report(tag+": dX matches the dense product",dx.Shape()==std::vector<uint32_t>({M,K})&&
+                                                     RelToMax(Download(dx),RefBackward(g,wd,M,N,K))<=tol);
+      }
+    }
+  }
+  {
     // 3-D input is flattened over the leading dims and reshaped back
     auto layer=MakeLayer(w,Dtype_e::Int8,Dtype_e::Float32,Scheme::PerChannel_e,16,stream,infer);
     std::vector<float> x3=Uniform(2*3*K,-1.0f,1.0f,202);
@@ -149,7 +179,7 @@ int main(int argc,char **argv)
   {
     CAIF_CudaStream null_stream=CAIF_CudaStream::Wrap(nullptr);
     Report("zero dims throw",Throws([&]{CAIF_DeviceFrozenLinear<float,int8_t> l(0,8,null_stream);},"must be > 0"));
-    Report("float storage cells are rejected",Throws([&]{CAIF_DeviceFrozenLinearFactory::Create(K,N,Dtype_e::Float32,null_stream);},"Int8 and Int4"));
+    Report("float storage cells are built",CAIF_DeviceFrozenLinearFactory::Create(K,N,Dtype_e::Float32,null_stream)->Description()=="FrozenLinear(16,8,fp32)");
     CAIF_DeviceFrozenLinear<caif_bf16_t,caif_int4_packed_t> l(K,N,null_stream);
     Report("defaults: group 128, cache hint true, per-tensor scheme",l.GroupSize()==128&&l.CacheFP32()==true&&
                                                                     l.Int8Scheme()==Scheme::PerTensor_e&&
