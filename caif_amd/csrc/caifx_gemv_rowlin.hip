@@ -71,6 +71,7 @@ struct RowArgs {
   int xpitch;           // staged activations: elements per row (cpr * k-per-chunk)
   int digits;           // int8, one activation row: take the integer-matrix-core kernel
   int round_x;          // that kernel only: activations pass through this dtype first (caifx_dtype), -1 = they are of it already
+  int slices;           // its form for K > 4096: parts a weight row is cut into (2 or 4), 0 otherwise
 };
 
 template <typename CT, typename XT>
@@ -817,6 +818,195 @@ __global__ __launch_bounds__(kDigitWaves * 64) void rowlin_int8_digits_kernel(Ro
 }
 
 
+// The same for reductions of 4097..16384 (a down projection at decode time).  The row no longer fits one wave's
+// registers, so the 16 waves of a workgroup split it: wave w takes slice w % nsl of every row of row group w / nsl,
+// a slice being `cps` <= 4 chunks of 1 KiB (the last slice may have fewer), and keeps that slice's digit planes in
+// registers for the whole kernel.  The power-of-two unit is taken per slice.  The nsl partial sums of a row meet in
+// LDS after the loop and are added in slice order.  a.cpr = chunks per row (K / 1024 <= 16), a.slices = nsl (2 or
+// 4), a.waves_per_class = row groups per residue class (a multiple of 16 / nsl).
+template <typename XT, bool kVec>
+__global__ __launch_bounds__(kDigitWaves * 64) void rowlin_int8_digits_long_kernel(RowArgs a)
+{
+  constexpr int CPS = 4;                  // chunks per slice at most
+  constexpr int D = 2;                    // row slices in the ring
+  __shared__ float mx[16][16];                                      // per chunk: max |x'| of every diagonal element
+  __shared__ __attribute__((aligned(16))) i32x4_t dig[16][3][64];   // [chunk][digit][lane]
+  __shared__ float red[kDigitWaves][64];                             // per wave: partial sums of its rows
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int nsl = a.slices;
+  const int cps = (a.cpr + nsl - 1) / nsl;
+  const int slice = wave % nsl;
+  const int groups_per_block = kDigitWaves / nsl;
+  const int grp = blockIdx.x * groups_per_block + wave / nsl;       // row group index over all classes
+  const int cls = (blockIdx.x * groups_per_block) / a.waves_per_class;
+  const int64_t i0 = static_cast<int64_t>(grp - cls * a.waves_per_class) * a.rows_per_wave;
+  const int64_t V = a.row_stride;
+  int nrows = 0;
+  {
+    const int64_t first = cls + V * i0;
+    if (first < a.N) {
+      const int64_t avail = (a.N - first + V - 1) / V;
+      nrows = static_cast<int>(avail < a.rows_per_wave ? avail : a.rows_per_wave);
+    }
+  }
+  const int64_t row_bytes = a.K;
+  const int first_chunk = slice * cps;
+  int my_chunks = a.cpr - first_chunk;                               // chunks of this wave's slice
+  my_chunks = my_chunks < 0 ? 0 : (my_chunks > cps ? cps : my_chunks);
+
+  // the activations and scales of chunk `wave` are requested before the first weight rows (see the kernel above)
+  float xv[16];
+  floatx4_t scv[4];
+  const bool has_chunk = wave < a.cpr;
+  if (has_chunk) {
+    const XT *xg = static_cast<const XT *>(a.x) + (wave * 64 + lane) * 16;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) xv[t] = to_f32<XT>(xg[t]);
+    if (a.round_x == CAIFX_BF16) {
+#pragma unroll
+      for (int t = 0; t < 16; ++t) xv[t] = round_through<bf16_t>(xv[t]);
+    } else if (a.round_x == CAIFX_F16) {
+#pragma unroll
+      for (int t = 0; t < 16; ++t) xv[t] = round_through<f16_t>(xv[t]);
+    }
+    if constexpr (kVec) {
+      const float *sp = static_cast<const float *>(a.scales);
+      const int idx = static_cast<int>((static_cast<int64_t>(cls) * a.K + (wave * 64 + lane) * 16) % a.period);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        int i = idx + 4 * q;
+        if (i >= a.period) i -= a.period;
+        scv[q] = *reinterpret_cast<const floatx4_t *>(sp + i);
+      }
+    }
+  }
+  float s_scalar = 1.0f;
+  if constexpr (!kVec) {
+    if (a.scales) s_scalar = static_cast<const float *>(a.scales)[0];
+  }
+
+  const uint8_t *wp = a.wq + (cls + V * i0) * row_bytes + first_chunk * 1024 + lane * 16;
+  const int64_t rstep = V * row_bytes;
+  i32x4_t w[D][CPS];
+  // unconditional loads: a row past the wave's range, or a chunk past the slice, reads the activation row
+  const uint8_t *wdummy = static_cast<const uint8_t *>(a.x) + lane * 16;
+  auto issue = [&](int d, int r) {
+    const uint8_t *wsrc = r < nrows ? wp + r * rstep : wdummy;
+#pragma unroll
+    for (int c = 0; c < CPS; ++c) w[d][c] = *reinterpret_cast<const i32x4_t *>(c < my_chunks ? wsrc + c * 1024 : wdummy);
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d) issue(d, d);
+
+  if (has_chunk) {
+    if constexpr (kVec) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) xv[4 * q + t] *= scv[q][t];
+    }
+    float m = 0.0f;
+    bool finite = true;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      m = fmaxf(m, fabsf(xv[t]));
+      finite = finite && fabsf(xv[t]) <= 3.4028235e38f;
+    }
+    m = finite ? m : __builtin_inff();
+    m = fmaxf(m, __shfl_xor(m, 16));
+    m = fmaxf(m, __shfl_xor(m, 32));
+    if (lane < 16) mx[wave][lane] = m;
+  }
+  __syncthreads();
+
+  // unit of diagonal element i within slice sl: the largest |x'| of the slice's chunks maps into [32, 64]
+  auto slice_max = [&](int sl) {
+    float m = 0.0f;
+    for (int c = sl * cps; c < (sl + 1) * cps && c < a.cpr; ++c) m = fmaxf(m, mx[c][lane & 15]);
+    return m;
+  };
+  auto unit_of = [&](float m) {
+    int e = 0;
+    (void)frexpf(m, &e);
+    return (m > 0.0f && m <= 3.4028235e38f) ? ldexpf(1.0f, e - 6) : 1.0f;
+  };
+  bool poisoned;       // the same in every wave of the workgroup
+  {
+    float m = 0.0f;
+    for (int c = 0; c < a.cpr; ++c) m = fmaxf(m, mx[c][lane & 15]);
+    poisoned = __any(!(m <= 3.4028235e38f));
+  }
+  if (has_chunk) {
+    const float unit_c = poisoned ? 1.0f : unit_of(slice_max(wave / cps));
+    const float inv14 = 16384.0f / unit_c;
+    i32x4_t d0, d1, d2;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      int e0[4], e1[4], e2[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int b = __builtin_bit_cast(int, __builtin_fmaf(xv[4 * q + t], inv14, 12582912.0f));
+        e2[t] = __builtin_amdgcn_sbfe(b, 0, 7);
+        e1[t] = __builtin_amdgcn_sbfe(b + 64, 7, 7);
+        e0[t] = __builtin_amdgcn_sbfe(b + 64 + 8192, 14, 8);
+      }
+      d0[q] = static_cast<int>(pack_low_bytes(e0[0], e0[1], e0[2], e0[3]));
+      d1[q] = static_cast<int>(pack_low_bytes(e1[0], e1[1], e1[2], e1[3]));
+      d2[q] = static_cast<int>(pack_low_bytes(e2[0], e2[1], e2[2], e2[3]));
+    }
+    dig[wave][0][lane] = d0;
+    dig[wave][1][lane] = d1;
+    dig[wave][2][lane] = d2;
+  }
+  __syncthreads();
+  const float unit = poisoned ? 1.0f : unit_of(slice_max(slice));
+  i32x4_t xb[CPS][3];
+#pragma unroll
+  for (int c = 0; c < CPS; ++c)
+#pragma unroll
+    for (int d = 0; d < 3; ++d) xb[c][d] = c < my_chunks ? dig[first_chunk + c][d][lane] : i32x4_t{0, 0, 0, 0};
+  const float u0 = unit * s_scalar, u1 = u0 * (1.0f / 128.0f), u2 = u0 * (1.0f / 16384.0f);
+  const int tsel = lane & 3;
+  const bool is_diag = (lane >> 4) == ((lane & 15) >> 2);
+
+  float res = 0.0f;          // lane r: this slice's share of the result of the wave's row r
+  for (int r0 = 0; r0 < nrows; r0 += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int r = r0 + d;
+      if (r < nrows) {
+        i32x4_t s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0}, s2 = {0, 0, 0, 0};
+#pragma unroll
+        for (int c = 0; c < CPS; ++c) {
+          s0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[d][c], xb[c][0], s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[d][c], xb[c][1], s1, 0, 0, 0);
+          s2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[d][c], xb[c][2], s2, 0, 0, 0);
+        }
+        int p0 = s0[0], p1 = s1[0], p2 = s2[0];
+        p0 = tsel == 1 ? s0[1] : p0;  p1 = tsel == 1 ? s1[1] : p1;  p2 = tsel == 1 ? s2[1] : p2;
+        p0 = tsel == 2 ? s0[2] : p0;  p1 = tsel == 2 ? s1[2] : p1;  p2 = tsel == 2 ? s2[2] : p2;
+        p0 = tsel == 3 ? s0[3] : p0;  p1 = tsel == 3 ? s1[3] : p1;  p2 = tsel == 3 ? s2[3] : p2;
+        float v = static_cast<float>(p0) * u0;
+        v = __builtin_fmaf(static_cast<float>(p1), u1, v);
+        v = __builtin_fmaf(static_cast<float>(p2), u2, v);
+        v = wave_sum_hi(is_diag ? v : 0.0f);
+        res = lane_insert(res, v, r);
+      }
+      issue(d, r + D);
+    }
+  }
+  red[wave][lane] = res;
+  __syncthreads();
+  if (slice == 0 && lane < nrows) {
+    float v = res;
+    for (int sl = 1; sl < nsl; ++sl) v += red[wave + sl][lane];
+    static_cast<float *>(a.y)[cls + V * (i0 + lane)] = poisoned ? __builtin_nanf("") : v;
+  }
+}
+
+
 // ------------------------------------------------------------------ int8, exact
 // kVec: per-channel scales (period > 1) cached in registers per residue class.
 template <typename CT, typename XT, int MT, bool kVec, int CPR>
@@ -956,6 +1146,10 @@ int launch_int4(const RowArgs &ra, hipStream_t s)
     if (full && ra.cpr == 1) return launch_int4_fast<CT, MT, 1>(ra, s);
     if (full && ra.cpr == 2) return launch_int4_fast<CT, MT, 2>(ra, s);
     if (full && ra.cpr == 4) return launch_int4_fast<CT, MT, 4>(ra, s);
+    if constexpr (MT == 1) {      // long reductions with one activation row (a down projection at decode time)
+      if (full && ra.cpr == 7) return launch_int4_fast<CT, MT, 7>(ra, s);
+      if (full && ra.cpr == 8) return launch_int4_fast<CT, MT, 8>(ra, s);
+    }
   }
   const size_t lds = static_cast<size_t>((MT * (ra.xpitch >> 7) + 3) & ~3) * 4 + static_cast<size_t>(MT) * ra.xpitch * 2;
   const unsigned grid = static_cast<unsigned>((ra.total_waves + 3) / 4);
@@ -974,6 +1168,11 @@ template <typename CT, typename XT, int MT, bool kVec>
 int launch_int8(const RowArgs &ra, hipStream_t s)
 {
   if constexpr (MT == 1) {
+    if (ra.digits && ra.slices > 0) {
+      hipLaunchKernelGGL((rowlin_int8_digits_long_kernel<XT, kVec>),
+                         dim3(static_cast<unsigned>(ra.total_waves / (kDigitWaves / ra.slices))), dim3(kDigitWaves * 64), 0, s, ra);
+      return launch_status();
+    }
     if (ra.digits) {
       if (ra.cpr == 1) return launch_int8_digits<XT, kVec, 1>(ra, s);
       if (ra.cpr == 2) return launch_int8_digits<XT, kVec, 2>(ra, s);
@@ -1089,7 +1288,9 @@ int rowlin_forward(const GemmArgs &g, hipStream_t s)
     ra.waves_per_class = ra.total_waves;
     if (static_cast<size_t>(mt) * ra.xpitch * 2 + 4096 > 64 * 1024) return CAIFX_ERR_UNSUPPORTED;
   } else {
-    if (g.K % 16 != 0 || g.K > 4096) return CAIFX_ERR_UNSUPPORTED;
+    // one activation row and 4096 < K <= 16384: the integer-matrix-core kernel with the row split among waves
+    const bool long_digits = g.M == 1 && g.K > 4096 && g.K <= 16384 && g.K % 1024 == 0 && g.y_dtype == CAIFX_F32;
+    if (g.K % 16 != 0 || (g.K > 4096 && !long_digits)) return CAIFX_ERR_UNSUPPORTED;
     ra.cpr = static_cast<int>((g.K + 1023) / 1024);
     ra.xpitch = ra.cpr * 1024;
     if (!g.w.scales || g.w.scale_period == 1) {
@@ -1105,7 +1306,25 @@ int rowlin_forward(const GemmArgs &g, hipStream_t s)
     }
     const int64_t rows_class = (g.N + ra.row_stride - 1) / ra.row_stride;
     const int rb = ra.cpr == 1 ? 8 : (ra.cpr == 2 ? 4 : 2);
-    const bool digits = g.M == 1 && g.K % 1024 == 0 && (ra.cpr == 1 || ra.cpr == 2 || ra.cpr == 4) && g.y_dtype == CAIFX_F32;
+    const bool digits = long_digits || (g.M == 1 && g.K % 1024 == 0 && (ra.cpr == 1 || ra.cpr == 2 || ra.cpr == 4) && g.y_dtype == CAIFX_F32);
+    if (long_digits) {
+      // wave w of a workgroup takes slice w % slices of the rows of row group w / slices; waves_per_class and
+      // total_waves count row groups here
+      ra.slices = ra.cpr > 8 ? 4 : 2;
+      ra.digits = 1;
+      ra.round_x = g.x_dtype != g.compute_dtype ? g.compute_dtype : -1;
+      const int groups_per_block = kDigitWaves / ra.slices;
+      const int64_t cus = compute_unit_count();
+      ra.rows_per_wave = 1;
+      while (ra.rows_per_wave < 64 &&
+             ra.row_stride * (((rows_class + ra.rows_per_wave - 1) / ra.rows_per_wave + groups_per_block - 1) / groups_per_block) > cus)
+        ++ra.rows_per_wave;
+      ra.waves_per_class = static_cast<int>((rows_class + ra.rows_per_wave - 1) / ra.rows_per_wave);
+      ra.waves_per_class = (ra.waves_per_class + groups_per_block - 1) / groups_per_block * groups_per_block;
+      ra.total_waves = ra.waves_per_class * ra.row_stride;
+      if (g.compute_dtype == CAIFX_BF16) return pick_xt<bf16_t>(ra, g.x_dtype, kind, s);
+      return pick_xt<f16_t>(ra, g.x_dtype, kind, s);
+    }
     // the integer-matrix-core kernel is light on registers and arithmetic: four waves per SIMD measured best
     ra.rows_per_wave = digits ? pick_rows_per_wave(g.N, 1, 4096) : pick_rows_per_wave(g.N, kind == 2 ? 2 * rb : rb);
     if (digits) {

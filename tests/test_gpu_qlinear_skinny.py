@@ -56,10 +56,13 @@ def test_decode_full_width_m1(orc, kind):
 
 
 @pytest.mark.parametrize("kind", ["int4", "int8pc", "int8pt"])
-@pytest.mark.parametrize("N,K,M", [(4096, 14336, 1), (4096, 14336, 16), (1024, 8192, 4), (528, 11008, 9), (640, 4224, 24)])
+@pytest.mark.parametrize("N,K,M", [(4096, 14336, 1), (4096, 14336, 16), (1024, 8192, 4), (528, 11008, 9), (640, 4224, 24),
+                                   (2048, 8192, 1), (1024, 11264, 1), (1536, 5120, 1), (512, 16384, 1), (1027, 9216, 1)])
 def test_reductions_longer_than_one_workgroup_covers(orc, kind, N, K, M):
     # the FFN down projection (N = 4096, K = 14336) and other K > 4096: the 16-row decode kernel cuts the
-    # reduction into slices of 4096 (the last one shorter) whose sums meet in the workspace
+    # reduction into slices of 4096 (the last one shorter) whose sums meet in the workspace; with one activation
+    # row the row-streaming kernels split a weight row among the waves of a workgroup (int8: 2 or 4 slices of up
+    # to 4 KiB, the last one shorter or empty; int4: 7 or 8 chunks per wave)
     rng = np.random.default_rng(N + K + M)
     _check(orc, rng, M, N, K, kind, cd=2, xd=2)
 
