@@ -18,9 +18,9 @@
 //         vector of period P is addressed by the flat index n*K + k modulo P; rows n with equal
 //         n mod V, V = P / gcd(K mod P, P), see the same scales along k, so a workgroup only visits
 //         rows of one residue class, stages that class's K scales in LDS once and forms
-//         x'[m][k] = x[m][k] * scale[k] in fp32.  x' is split into three signed 7-bit digit planes
-//         relative to a power-of-two unit per activation row and wave (x' ~ unit * (d0 + d1/128 +
-//         d2/16384), error <= unit * 2^-15); the three exact int32 sums are combined in fp32 per block.
+//         x'[m][k] = x[m][k] * scale[k] in fp32.  x' is split into three signed 8-bit digit planes
+//         relative to a power-of-two unit per activation row and wave (x' ~ unit * (d0 + d1/256 +
+//         d2/65536), |d0| <= 32, error <= unit * 2^-17); the three exact int32 sums are combined in fp32 per block.
 //         The weight is therefore never rounded to the compute dtype: results differ from the
 //         dequantise-then-cast reference by that rounding (a few 1e-3 of the largest output), like int4.
 // After the last group every wave holds a partial 16x16 tile; the 16 partials are added through LDS
@@ -280,7 +280,7 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
   // int8: digit planes of x' = x * scale as A operands of the integer matrix core, dg[step][plane];
   // step t covers k = (g0 + t/2)*128 + (t%2)*64 + q*16 .. +16 of activation row j
   constexpr int kSteps = 2 * GPW;
-  constexpr int kPlanes = 3;              // 2 would give 14-bit activations; the third plane costs 4 of 12 MFMAs per block
+  constexpr int kPlanes = 3;              // signed 8-bit digits: x' to 2^-21 of the largest |x'| of the row in this wave's k range
   i32x4_t dg[kInt4 ? 1 : kSteps][kPlanes];
   float ur[4] = {1.0f, 1.0f, 1.0f, 1.0f};     // unit of the activation rows 4q..4q+3 this lane holds results of
   bool poison[4] = {false, false, false, false};   // those rows have a non-finite scaled activation in this wave's k range
@@ -312,6 +312,8 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] *= sc4[i];
     };
+    // first pass: x' = x * scale, kept in registers for the second pass; the largest |x'| and whether all are finite
+    float xp[kSteps][16];
     float mx = 0.0f;
     bool finite = true;
 #pragma unroll
@@ -322,6 +324,7 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
         xprime4(t, c, v);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+          xp[t][4 * c + i] = v[i];
           mx = fmaxf(mx, fabsf(v[i]));                       // ignores a NaN
           finite = finite && fabsf(v[i]) <= 3.4028235e38f;    // false for NaN and infinities
         }
@@ -336,33 +339,31 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
     for (int r = 0; r < 4; ++r) poison[r] = __shfl(bad, 4 * q + r) != 0;
     int e = 0;
     (void)frexpf(mx, &e);                     // mx = f * 2^e, f in [0.5, 1)
-    const float unit = mx > 0.0f ? ldexpf(1.0f, e - 6) : 1.0f;    // |x'| / unit <= 64
-    const float inv14 = 16384.0f / unit;      // exact: a power of two
+    const float unit = mx > 0.0f ? ldexpf(1.0f, e - 5) : 1.0f;    // |x'| / unit < 32
+    const float inv16 = 65536.0f / unit;      // exact: a power of two
+    // second pass: n = round(x' / unit * 2^16) sits in the low mantissa bits of b = x' * inv16 + 1.5 * 2^23
+    // (|n| <= 2^21), and n = 2^16 d0 + 2^8 d1 + d2 with d1, d2 in [-128, 127]: d2 is byte 0 of b, d1 byte 1 of
+    // b + 0x80, d0 byte 2 of b + 0x8080 less the 0x40 that the constant leaves there (adding 0xC00000 removes it).
+    // One byte permute per pair of values and one per plane gather the bytes of four values.
+    auto gather = [&](uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3, uint32_t sel) __attribute__((always_inline)) {
+      const uint32_t lo = __builtin_amdgcn_perm(a1, a0, sel);
+      const uint32_t hi = __builtin_amdgcn_perm(a3, a2, sel);
+      return static_cast<int>(__builtin_amdgcn_perm(hi, lo, 0x05040100u));
+    };
 #pragma unroll
     for (int t = 0; t < kSteps; ++t) {
-      // n = round(x' / unit * 2^14) as the low mantissa bits of x' * inv14 + 1.5 * 2^23 (|n| <= 2^20);
-      // n = 2^14 d0 + 2^7 d1 + d2 with d1, d2 in [-64, 63]
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        float v[4];
-        xprime4(t, c, v);
-        int e0[4], e1[4], e2[4];
+        uint32_t b0[4], b1[4], b2[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int b = __builtin_bit_cast(int, __builtin_fmaf(v[i], kPlanes == 3 ? inv14 : inv14 * (1.0f / 128.0f), 12582912.0f));
-          if constexpr (kPlanes == 3) {
-            e2[i] = __builtin_amdgcn_sbfe(b, 0, 7);
-            e1[i] = __builtin_amdgcn_sbfe(b + 64, 7, 7);
-            e0[i] = __builtin_amdgcn_sbfe(b + 64 + 8192, 14, 8);
-          } else {
-            e2[i] = 0;
-            e1[i] = __builtin_amdgcn_sbfe(b, 0, 7);
-            e0[i] = __builtin_amdgcn_sbfe(b + 64, 7, 8);
-          }
+          b0[i] = __builtin_bit_cast(uint32_t, __builtin_fmaf(xp[t][4 * c + i], inv16, 12582912.0f));
+          b1[i] = b0[i] + 0x80u;
+          b2[i] = b0[i] + 0xC08080u;
         }
-        dg[t][0][c] = static_cast<int>(pack_low_bytes(e0[0], e0[1], e0[2], e0[3]));
-        dg[t][1][c] = static_cast<int>(pack_low_bytes(e1[0], e1[1], e1[2], e1[3]));
-        if constexpr (kPlanes == 3) dg[t][2][c] = static_cast<int>(pack_low_bytes(e2[0], e2[1], e2[2], e2[3]));
+        dg[t][0][c] = gather(b2[0], b2[1], b2[2], b2[3], 0x0c0c0602u);
+        dg[t][1][c] = gather(b1[0], b1[1], b1[2], b1[3], 0x0c0c0501u);
+        dg[t][2][c] = gather(b0[0], b0[1], b0[2], b0[3], 0x0c0c0400u);
       }
     }
 #pragma unroll
@@ -411,13 +412,13 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
               const i32x4_t bw = __builtin_bit_cast(i32x4_t, w[d][t]);
               s0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[t][0], bw, s0, 0, 0, 0);
               s1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[t][1], bw, s1, 0, 0, 0);
-              if constexpr (kPlanes == 3) s2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[t][2], bw, s2, 0, 0, 0);
+              s2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[t][2], bw, s2, 0, 0, 0);
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               float v = static_cast<float>(s0[r]);
-              v = __builtin_fmaf(static_cast<float>(s1[r]), 1.0f / 128.0f, v);
-              if constexpr (kPlanes == 3) v = __builtin_fmaf(static_cast<float>(s2[r]), 1.0f / 16384.0f, v);
+              v = __builtin_fmaf(static_cast<float>(s1[r]), 1.0f / 256.0f, v);
+              v = __builtin_fmaf(static_cast<float>(s2[r]), 1.0f / 65536.0f, v);
               tot[u][r] = poison[r] ? __builtin_nanf("") : v * ur[r];
             }
           }

@@ -121,12 +121,14 @@ __global__ void absmax_columns_kernel(const float *__restrict__ in, uint32_t *__
 {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= cols) return;
-  const int r0 = blockIdx.y * kRowChunk;
-  const int r1 = r0 + kRowChunk < rows ? r0 + kRowChunk : rows;
   float m = 0.0f;
-  for (int r = r0; r < r1; ++r) {
-    float v = fabsf(in[static_cast<int64_t>(r) * cols + c]);
-    if (v > m) m = v;
+  // chunks of rows are strided over gridDim.y, which the launch caps at the grid limit
+  for (int64_t r0 = static_cast<int64_t>(blockIdx.y) * kRowChunk; r0 < rows; r0 += static_cast<int64_t>(gridDim.y) * kRowChunk) {
+    const int64_t r1 = r0 + kRowChunk < rows ? r0 + kRowChunk : rows;
+    for (int64_t r = r0; r < r1; ++r) {
+      float v = fabsf(in[r * cols + c]);
+      if (v > m) m = v;
+    }
   }
   if (m > 0.0f) atomicMax(acc + c, __float_as_uint(m));
 }
@@ -466,8 +468,9 @@ int caifx_quantize_int8_per_channel(const float *input, void *output, void *scal
     hipLaunchKernelGGL(absmax_columns_x4_kernel, dim3(grid_for(cols / 4, 64), (rows + kRowChunk - 1) / kRowChunk), dim3(64),
                        0, s, input, static_cast<uint32_t *>(scales), rows, cols);
   else
-    hipLaunchKernelGGL(absmax_columns_kernel, dim3(grid_for(cols), (rows + kRowChunk - 1) / kRowChunk), dim3(kBlock), 0,
-                       s, input, static_cast<uint32_t *>(scales), rows, cols);
+    hipLaunchKernelGGL(absmax_columns_kernel,
+                       dim3(grid_for(cols), (rows + kRowChunk - 1) / kRowChunk > 65535 ? 65535 : (rows + kRowChunk - 1) / kRowChunk),
+                       dim3(kBlock), 0, s, input, static_cast<uint32_t *>(scales), rows, cols);
   hipLaunchKernelGGL(finalize_int8_scale_kernel, dim3(grid_for(cols)), dim3(kBlock), 0, s,
                      static_cast<float *>(scales), cols);
   if (x4)

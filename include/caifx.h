@@ -178,7 +178,8 @@ CAIFX_API int caifx_qlinear_backward_input_add(int64_t M, int64_t N, int64_t K,
  * backward != 0 asks for caifx_qlinear_backward_input.  Nonzero for 16-bit compute types when the result has
  * fewer 128 x 128 tiles than the chip has compute units: up to 8 workgroups then share a tile's reduction through
  * fp32 partial tiles in the workspace (16-byte aligned) and a second launch adds them in a fixed order (results do
- * not depend on scheduling).  The fp32 compute type does the same for up to 128 rows.  With a smaller or null
+ * not depend on scheduling).  The fp32 compute type does the same for up to 128 rows, and the forward with up to
+ * 32 rows and K > 4096 cuts the reduction into slices of 4096 whose sums meet there.  With a smaller or null
  * workspace the calls run without that sharing, only slower, and the sums are formed in a different order, so
  * the last bits of a result may differ between a call with and a call without the workspace. */
 CAIFX_API size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtype, int compute_dtype,

@@ -51,6 +51,23 @@ def test_two_calls_second_smaller_match_the_workspace_form(orc, kind, cd, xd):
         assert max_rel_err(host(y), orc.frozen_linear_forward(host(x), ow, cd)) <= tol
 
 
+@pytest.mark.parametrize("kind", ["int4", "int8pc"])
+def test_long_reduction_slices_meet_in_the_static_buffer(orc, kind):
+    # K > 4096 with up to 32 rows: the 16-row decode kernel's slices of the reduction use the same buffer
+    rng = np.random.default_rng(47)
+    N, K = 1024, 8192
+    ow, dw = make_weight(orc, rng, N, K, kind)
+    for M in (16, 24, 5):
+        assert 0 < _need(M, dw, 2, 2) <= SCRATCH_BYTES
+        x = dev_as(rng.normal(0, 1, (M, K)), 2)
+        st, y = _static(x, dw, 2)
+        assert st == 0, capi.status_string(st)
+        want = T.qlinear_forward(x, dw, 2)
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), (kind, M)
+        assert max_rel_err(host(y), orc.frozen_linear_forward(host(x), ow, 2)) <= 1e-2
+
+
 def test_shapes_without_scratch_run_and_oversized_ones_are_refused(orc):
     rng = np.random.default_rng(43)
     ow, dw = make_weight(orc, rng, 4096, 4096, "int4")
