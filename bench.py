@@ -322,6 +322,16 @@ def quantise_rows(torch, T, dev, gen):
         ms = timed(fn)
         out[name] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                      "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    # the dequantisers (checkpoint export path): codes + scales in, fp32 out
+    q8, s8 = T.quantize_int8(ws[0], per_channel=True)
+    p4, s4 = T.quantize_int4_per_group(ws[0], 128)
+    for name, fn, nbytes in (
+            ("dequant_int8_per_channel_4096x14336", lambda: T.dequantize_int8(q8, s8, per_channel=True), n + cols * 4 + n * 4),
+            ("dequant_int4_group128_4096x14336", lambda: T.dequantize_int4_per_group(p4, s4, n, 128),
+             n // 2 + n // 128 * 2 + n * 4)):
+        ms = timed(fn)
+        out[name] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                     "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     return {"quantise_ops": out}
 
 

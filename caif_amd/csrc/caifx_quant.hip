@@ -267,6 +267,44 @@ __global__ void dequantize_int8_kernel(const int8_t *__restrict__ in, float *__r
   }
 }
 
+// Four consecutive codes per thread (4-byte aligned codes, 16-byte aligned output): one dword in, one 16-byte
+// store out, consecutive lanes on consecutive addresses.  The scale vector has period `period`, a multiple of 4
+// that divides n, so the four scales of a thread are consecutive and do not wrap (period 1: one scale).  Same
+// product per element as dequantize_int8_kernel.
+__global__ void dequantize_int8_x4_kernel(const int8_t *__restrict__ in, float *__restrict__ out,
+                                          const float *__restrict__ scales, int64_t n4, int period)
+{
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n4) return;
+  const uint32_t w = reinterpret_cast<const uint32_t *>(in)[i];
+  floatx4_t s;
+  if (period == 1) {
+    const float one = scales[0];
+    s = floatx4_t{one, one, one, one};
+  } else {
+    s = *reinterpret_cast<const floatx4_t *>(scales + (i * 4) % period);
+  }
+  float e[4];
+  int8x4_to_f32(w, e);
+  reinterpret_cast<floatx4_t *>(out)[i] = floatx4_t{e[0] * s[0], e[1] * s[1], e[2] * s[2], e[3] * s[3]};
+}
+
+int launch_dequantize_int8(const int8_t *in, float *out, const float *scales, int64_t n, int period, hipStream_t s)
+{
+  const bool vec = aligned_to(in, 4) && aligned_to(out, 16) &&
+                   (period == 1 || (period % 4 == 0 && n % period == 0 && aligned_to(scales, 16)));
+  const int64_t body = vec ? n / 4 * 4 : 0;
+  if (body > 0)
+    hipLaunchKernelGGL(dequantize_int8_x4_kernel, dim3(grid_for(body / 4)), dim3(kBlock), 0, s, in, out, scales, body / 4,
+                       period);
+  // a tail is left only with one scale (period 1) or when nothing went the vector way: n is a multiple of the
+  // period, so a period that is a multiple of 4 leaves none
+  if (body < n)
+    hipLaunchKernelGGL(dequantize_int8_kernel, dim3(grid_for((n - body + 3) / 4)), dim3(kBlock), 0, s, in + body,
+                       out + body, scales, n - body, period);
+  return launch_status();
+}
+
 // ------------------------------------------------------------------ int4 per-group
 // Fast path: each thread owns 8 consecutive elements (one dword of packed output); a team of
 // group_size/8 adjacent lanes owns one group and shares its max through wave shuffles.
@@ -446,9 +484,8 @@ int caifx_dequantize_int8_per_tensor(const void *input, float *output, const voi
 {
   if (n <= 0) return CAIFX_OK;
   if (!input || !output || !scale) return CAIFX_ERR_INVALID_ARGUMENT;
-  hipLaunchKernelGGL(dequantize_int8_kernel, dim3(grid_for((n + 3) / 4)), dim3(kBlock), 0, as_stream(stream),
-                     static_cast<const int8_t *>(input), output, static_cast<const float *>(scale), n, 1);
-  return launch_status();
+  return launch_dequantize_int8(static_cast<const int8_t *>(input), output, static_cast<const float *>(scale), n, 1,
+                                as_stream(stream));
 }
 
 int caifx_quantize_int8_per_channel(const float *input, void *output, void *scales, int rows, int cols,
@@ -489,9 +526,8 @@ int caifx_dequantize_int8_per_channel(const void *input, float *output, const vo
   if (rows <= 0 || cols <= 0) return CAIFX_OK;
   if (!input || !output || !scales) return CAIFX_ERR_INVALID_ARGUMENT;
   const int64_t n = static_cast<int64_t>(rows) * cols;
-  hipLaunchKernelGGL(dequantize_int8_kernel, dim3(grid_for((n + 3) / 4)), dim3(kBlock), 0, as_stream(stream),
-                     static_cast<const int8_t *>(input), output, static_cast<const float *>(scales), n, cols);
-  return launch_status();
+  return launch_dequantize_int8(static_cast<const int8_t *>(input), output, static_cast<const float *>(scales), n, cols,
+                                as_stream(stream));
 }
 
 int caifx_quantize_to_int4(const float *input, void *packed_output, void *scales_output,
