@@ -80,9 +80,10 @@ def main():
     copies8 = max(2, -(-512 * 2**20 // algorithmic_bytes("int8", 1)))
     W4 = [T.FrozenWeight(p4.clone(), T.W_INT4_GROUP, s4.clone(), N_DEC, K_DEC, 1, 128) for _ in range(copies4)]
     W8 = [T.FrozenWeight(q8.clone(), T.W_INT8, s8.clone(), N_DEC, K_DEC, N_DEC) for _ in range(copies8)]
-    X = {m: torch.empty(m, K_DEC, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16) for m in (1, 4, 16)}
-    Y = {m: torch.empty(m, N_DEC, device=dev) for m in (1, 4, 16)}
-    ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    # M = 1, 4, 16 are the configuration's rows; 32 rows (two 16-row tiles in one pass over the weight) is an extra row
+    X = {m: torch.empty(m, K_DEC, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16) for m in (1, 4, 16, 32)}
+    Y = {m: torch.empty(m, N_DEC, device=dev) for m in (1, 4, 16, 32)}
+    ws = torch.empty(4 << 20, dtype=torch.uint8, device=dev)      # partial sums of the 32-row kernel's two reduction slices
 
     def gemv(fw, m):
         T.qlinear_forward(X[m], fw, T.BF16, T.F32, out=Y[m], workspace=ws)
@@ -152,7 +153,7 @@ def main():
     L = 128
     per = {}
     for kind, Ws, nc in (("int4", W4, copies4), ("int8", W8, copies8)):
-        for m in (1, 4, 16):
+        for m in (1, 4, 16, 32):
             if m != 1 and args.no_extra:
                 continue
             g = capture(lambda i, Ws=Ws, nc=nc, m=m: gemv(Ws[i % nc], m), L)

@@ -114,8 +114,6 @@ size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtyp
   const size_t f32_bytes = mfma_f32_workspace_bytes(a, backward != 0);
   size_t bytes = mfma_workspace_bytes(a, backward != 0);
   if (!backward) {
-    // up to 32 rows go through the 16-row decode kernel, 16 rows at a time
-    if (a.M > 16 && a.M <= 32) a.M = 16;
     const size_t decode_bytes = mblock_workspace_bytes(a);
     if (decode_bytes > bytes) bytes = decode_bytes;
   }
@@ -153,11 +151,11 @@ static int forward_impl(int64_t M, int64_t N, int64_t K, const void *x, int x_dt
   // one or two rows: stream each weight row linearly and reduce per row; from three rows on the
   // matrix-core tiling (cost independent of M) is faster; both fall through when a shape does not fit
   st = CAIFX_ERR_UNSUPPORTED;
-  // fp32 compute.  int8 storage with up to 16 rows: the 16-row decode kernel on the integer matrix core (digit
+  // fp32 compute.  int8 storage with up to 32 rows: the row-block decode kernel on the integer matrix core (digit
   // planes of the fp32 activations); otherwise from two rows on the fp32 matrix-core kernel (40-43 us at
   // K = N = 4096 whatever M <= 32); the VALU decode kernel below takes 40-46 us for one row
   if (compute_dtype == CAIFX_F32) {
-    if (M <= 16 && w_kind == CAIFX_W_INT8) {
+    if (M <= 32 && w_kind == CAIFX_W_INT8) {
       st = mblock_forward(a, s);
       if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, y, y_dtype, M * N, stream);
     }
@@ -174,16 +172,20 @@ static int forward_impl(int64_t M, int64_t N, int64_t K, const void *x, int x_dt
     if (st == CAIFX_ERR_UNSUPPORTED) st = skinny_forward(a, s);
   }
   if (M > 16 && M <= 32) {
-    // 17..32 rows: two launches of the 16-row decode kernel (2 x 14-17 us at K = 4096, N = 4096..14336) beat
-    // the tiled GEMM, whose shortest launch is one tile's reduction (43 us int4, 68 us int8 at K = 4096)
-    GemmArgs c = a;
-    c.M = 16;
-    st = mblock_forward(c, s);
-    if (st == CAIFX_OK) {
-      c.M = M - 16;
-      c.x = static_cast<const char *>(x) + 16 * K * static_cast<int64_t>(dtype_size(x_dtype));
-      c.y = static_cast<char *>(y) + 16 * N * static_cast<int64_t>(dtype_size(y_dtype));
+    // 17..32 rows: the decode kernel with two tiles of 16 rows reads the weight once; without the workspace its
+    // reduction slices need, two launches of the 16-row form (2 x 14-17 us at K = 4096, N = 4096..14336) still
+    // beat the tiled GEMM, whose shortest launch is one tile's reduction (43 us int4, 68 us int8 at K = 4096)
+    st = mblock_forward(a, s);
+    if (st == CAIFX_ERR_UNSUPPORTED) {
+      GemmArgs c = a;
+      c.M = 16;
       st = mblock_forward(c, s);
+      if (st == CAIFX_OK) {
+        c.M = M - 16;
+        c.x = static_cast<const char *>(x) + 16 * K * static_cast<int64_t>(dtype_size(x_dtype));
+        c.y = static_cast<char *>(y) + 16 * N * static_cast<int64_t>(dtype_size(y_dtype));
+        st = mblock_forward(c, s);
+      }
     }
   }
   if (st == CAIFX_ERR_UNSUPPORTED) {

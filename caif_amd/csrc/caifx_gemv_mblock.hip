@@ -126,6 +126,9 @@ __device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d)
   return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
 }
 
+// row blocks between two additions of the waves' partial tiles
+constexpr int mb_reduce_blocks(bool int4, int mt) { return int4 && mt == 1 ? 4 : 2; }
+
 constexpr int kSegBlocks = 16;                         // row blocks between two flushes of the output staging buffer
 constexpr int kSegRows = kSegBlocks * 16;
 
@@ -139,9 +142,11 @@ constexpr int kSegRows = kSegBlocks * 16;
 // kF32 (int8 only): fp32 compute type.  The activations are not rounded to a 16-bit type: the digit planes are cut
 // from x * scale in fp32, read from memory in both passes over them instead of being kept in registers (CT then
 // only names a vector type nothing is stored in).
-// wq / scales: the weight; xrows / yrows: the first of the M <= 16 activation and result rows; slice: which part of
+// MT: tiles of 16 activation rows that share one pass over the weight (M <= 16 * MT); every weight fragment is
+// unpacked once and multiplied with each tile's operands.
+// wq / scales: the weight; xrows / yrows: the first of the M activation and result rows; slice: which part of
 // the reduction (see MbArgs).  Every thread of the workgroup makes the same calls (the body has barriers).
-template <typename CT, typename XT, bool kInt4, int GPW, bool kF32>
+template <typename CT, typename XT, bool kInt4, int GPW, bool kF32, int MT = 1>
 __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, const void *scales, const void *xrows,
                                             void *yrows, int M, int slice)
 {
@@ -150,11 +155,12 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
   constexpr int LPG = kInt4 ? 1 : 2;           // 16-byte loads per lane per 128-k group
   constexpr int LPR = GPW * LPG;               // ... per block of 16 weight rows
   constexpr int D = 2;                         // row blocks in the ring
-  constexpr int RBB = kInt4 ? 4 : 2;           // row blocks between two reductions (a multiple of D, divides kSegBlocks)
+  constexpr int RBB = mb_reduce_blocks(kInt4, MT);      // row blocks between two reductions (a multiple of D, divides kSegBlocks)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  float *partial = reinterpret_cast<float *>(smem);      // [RBB][16 waves][4][64]
-  float *ybuf = partial + RBB * kPartialFloats;          // [16 activation rows][kSegRows]
-  float *svec = ybuf + 16 * kSegRows;                    // int8 with a scale vector: [K]
+  float *partial = reinterpret_cast<float *>(smem);      // [RBB][MT][16 waves][4][64]
+  float *ybuf = partial + RBB * MT * kPartialFloats;     // [16 * MT activation rows][kSegRows]
+  float *svec = ybuf + 16 * MT * kSegRows;               // int8: the scale vector of this slice [slice k]; int4 with
+                                                         // MT > 1: the group-sum corrections [MT][GPW][16 waves][16]
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -199,18 +205,23 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
   // Order of the requests: this wave's slice of X and (int8) the scale vector first, they come from
   // L2 and are needed first; then the first weight blocks.  Loads return in order, so the prologue
   // runs while the weights are still on their way from HBM.
-  vec_t xa[GPW][4];
-  const XT *xg = static_cast<const XT *>(xrows) + static_cast<int64_t>(j < M ? j : M - 1) * a.K + kbase;
+  vec_t xa[MT][GPW][4];
+  const XT *xg[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+    xg[mt] = static_cast<const XT *>(xrows) + static_cast<int64_t>(16 * mt + j < M ? 16 * mt + j : M - 1) * a.K + kbase;
   if constexpr (!kF32) {
 #pragma unroll
-    for (int g = 0; g < GPW; ++g) {
-      const int gg = g0 + g < groups ? g0 + g : groups - 1;
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const int k = kInt4 ? gg * 128 + q * 32 + 8 * t : gg * 128 + (t >> 1) * 64 + q * 16 + 8 * (t & 1);
-        xa[g][t] = load_x8<CT, XT>(xg + k);
+      for (int g = 0; g < GPW; ++g) {
+        const int gg = g0 + g < groups ? g0 + g : groups - 1;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int k = kInt4 ? gg * 128 + q * 32 + 8 * t : gg * 128 + (t >> 1) * 64 + q * 16 + 8 * (t & 1);
+          xa[mt][g][t] = load_x8<CT, XT>(xg[mt] + k);
+        }
       }
-    }
   }
   // int8 scale vector of this residue class: svec[k] = scales[(cls*K + k) mod period], K <= 4096
   float s_one = 1.0f;
@@ -236,11 +247,13 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
 #pragma unroll
     for (int i = 0; i < 8; ++i) zero[i] = from_f32<CT>(0.0f);
 #pragma unroll
-    for (int g = 0; g < GPW; ++g) {
-      const bool live = g0 + g < groups && j < M;
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) xa[g][t] = live ? xa[g][t] : zero;
-    }
+      for (int g = 0; g < GPW; ++g) {
+        const bool live = g0 + g < groups && 16 * mt + j < M;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) xa[mt][g][t] = live ? xa[mt][g][t] : zero;
+      }
   }
   if constexpr (!kInt4) {
 #pragma unroll
@@ -252,47 +265,64 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
 
   // int4: the nibbles unpack in the order 0,4,1,5,2,6,3,7, so X is stored that way; and
   // cor = OFFSET * (sum of x over each group) for the four activation rows this lane holds results of
-  float cor[GPW][4];
+  // (one tile keeps them in registers; with more tiles they wait in LDS, a wave reads back only what it wrote)
+  float cor[MT == 1 ? GPW : 1][4];
+  float *corbuf = svec + wave * 16;
   if constexpr (kInt4) {
     vec_t ones;
 #pragma unroll
     for (int i = 0; i < 8; ++i) ones[i] = from_f32<CT>(1.0f);
 #pragma unroll
-    for (int g = 0; g < GPW; ++g) {
-      // the group sums come out of the matrix core in the layout of the results: X times a matrix of ones
-      floatx4_t xsum = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const vec_t v = xa[g][t];
-        xsum = Mfma16<CT>::run(v, ones, xsum);
-        vec_t p;
+      for (int g = 0; g < GPW; ++g) {
+        // the group sums come out of the matrix core in the layout of the results: X times a matrix of ones
+        floatx4_t xsum = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          p[2 * i] = v[i];
-          p[2 * i + 1] = v[i + 4];
+        for (int t = 0; t < 4; ++t) {
+          const vec_t v = xa[mt][g][t];
+          xsum = Mfma16<CT>::run(v, ones, xsum);
+          vec_t p;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            p[2 * i] = v[i];
+            p[2 * i + 1] = v[i + 4];
+          }
+          xa[mt][g][t] = p;
         }
-        xa[g][t] = p;
-      }
+        if constexpr (MT == 1) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) cor[g][r] = Mfma16<CT>::kOffset * xsum[r];
-    }
+          for (int r = 0; r < 4; ++r) cor[g][r] = Mfma16<CT>::kOffset * xsum[r];
+        } else if (j == 0) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) corbuf[(mt * GPW + g) * (kMbWaves * 16) + 4 * q + r] = Mfma16<CT>::kOffset * xsum[r];
+        }
+      }
+    if constexpr (MT > 1) __syncthreads();
   }
   // int8: digit planes of x' = x * scale as A operands of the integer matrix core, dg[step][plane];
   // step t covers k = (g0 + t/2)*128 + (t%2)*64 + q*16 .. +16 of activation row j
   constexpr int kSteps = 2 * GPW;
   constexpr int kPlanes = 3;              // signed 8-bit digits: x' to 2^-21 of the largest |x'| of the row in this wave's k range
-  i32x4_t dg[kInt4 ? 1 : kSteps][kPlanes];
-  float ur[4] = {1.0f, 1.0f, 1.0f, 1.0f};     // unit of the activation rows 4q..4q+3 this lane holds results of
-  bool poison[4] = {false, false, false, false};   // those rows have a non-finite scaled activation in this wave's k range
+  i32x4_t dg[kInt4 ? 1 : MT][kInt4 ? 1 : kSteps][kPlanes];
+  float ur[MT][4];            // unit of the activation rows 4q..4q+3 of each tile, which this lane holds results of
+  bool poison[MT][4];         // those rows have a non-finite scaled activation in this wave's k range
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      ur[mt][r] = 1.0f;
+      poison[mt][r] = false;
+    }
   if constexpr (!kInt4) {
     __syncthreads();       // svec is complete
-    // four consecutive x' values: quad c (0..3) of step t
-    auto xprime4 = [&](int t, int c, float (&v)[4]) {
+    // four consecutive x' values: quad c (0..3) of step t of tile mt
+    auto xprime4 = [&](int mt, int t, int c, float (&v)[4]) {
       const int g = t >> 1;
       const int gg = g0 + g < groups ? g0 + g : groups - 1;
       if constexpr (kF32) {
-        const bool live = g0 + g < groups && j < M;
-        const XT *px = xg + gg * 128 + (t & 1) * 64 + q * 16 + 4 * c;
+        const bool live = g0 + g < groups && 16 * mt + j < M;
+        const XT *px = xg[mt] + gg * 128 + (t & 1) * 64 + q * 16 + 4 * c;
         if constexpr (sizeof(XT) == 4) {
           const floatx4_t xv = *reinterpret_cast<const floatx4_t *>(px);
 #pragma unroll
@@ -304,7 +334,7 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
           for (int i = 0; i < 4; ++i) v[i] = live ? to_f32<XT>(h[i]) : 0.0f;
         }
       } else {
-        const vec_t xv = xa[g][2 * (t & 1) + (c >> 1)];
+        const vec_t xv = xa[mt][g][2 * (t & 1) + (c >> 1)];
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = to_f32<CT>(xv[4 * (c & 1) + i]);
       }
@@ -312,38 +342,6 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] *= sc4[i];
     };
-    // first pass: x' = x * scale, kept in registers for the second pass; the largest |x'| and whether all are finite
-    float xp[kSteps][16];
-    float mx = 0.0f;
-    bool finite = true;
-#pragma unroll
-    for (int t = 0; t < kSteps; ++t)
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        float v[4];
-        xprime4(t, c, v);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          xp[t][4 * c + i] = v[i];
-          mx = fmaxf(mx, fabsf(v[i]));                       // ignores a NaN
-          finite = finite && fabsf(v[i]) <= 3.4028235e38f;    // false for NaN and infinities
-        }
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));      // over the four k quarters: row j's largest |x'| in this wave's k range
-    // A NaN or an infinity among row j's scaled activations has no digits.  The reference's GEMM returns NaN or an
-    // infinity in every output of that activation row; here this wave's share of them, and so their sum, is NaN.
-    const int bad = (__ballot(!finite) >> j & 0x0001000100010001ull) != 0 ? 1 : 0;
-    mx = bad ? 1.0f : mx;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) poison[r] = __shfl(bad, 4 * q + r) != 0;
-    int e = 0;
-    (void)frexpf(mx, &e);                     // mx = f * 2^e, f in [0.5, 1)
-    const float unit = mx > 0.0f ? ldexpf(1.0f, e - 5) : 1.0f;    // |x'| / unit < 32
-    const float inv16 = 65536.0f / unit;      // exact: a power of two
-    // second pass: n = round(x' / unit * 2^16) sits in the low mantissa bits of b = x' * inv16 + 1.5 * 2^23
-    // (|n| <= 2^21), and n = 2^16 d0 + 2^8 d1 + d2 with d1, d2 in [-128, 127]: d2 is byte 0 of b, d1 byte 1 of
-    // b + 0x80, d0 byte 2 of b + 0x8080 less the 0x40 that the constant leaves there (adding 0xC00000 removes it).
     // One byte permute per pair of values and one per plane gather the bytes of four values.
     auto gather = [&](uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3, uint32_t sel) __attribute__((always_inline)) {
       const uint32_t lo = __builtin_amdgcn_perm(a1, a0, sel);
@@ -351,23 +349,58 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
       return static_cast<int>(__builtin_amdgcn_perm(hi, lo, 0x05040100u));
     };
 #pragma unroll
-    for (int t = 0; t < kSteps; ++t) {
+    for (int mt = 0; mt < MT; ++mt) {
+      // first pass: x' = x * scale, kept in registers for the second pass; the largest |x'| and whether all are finite
+      float xp[kSteps][16];
+      float mx = 0.0f;
+      bool finite = true;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        uint32_t b0[4], b1[4], b2[4];
+      for (int t = 0; t < kSteps; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          b0[i] = __builtin_bit_cast(uint32_t, __builtin_fmaf(xp[t][4 * c + i], inv16, 12582912.0f));
-          b1[i] = b0[i] + 0x80u;
-          b2[i] = b0[i] + 0xC08080u;
+        for (int c = 0; c < 4; ++c) {
+          float v[4];
+          xprime4(mt, t, c, v);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            xp[t][4 * c + i] = v[i];
+            mx = fmaxf(mx, fabsf(v[i]));                       // ignores a NaN
+            finite = finite && fabsf(v[i]) <= 3.4028235e38f;    // false for NaN and infinities
+          }
         }
-        dg[t][0][c] = gather(b2[0], b2[1], b2[2], b2[3], 0x0c0c0602u);
-        dg[t][1][c] = gather(b1[0], b1[1], b1[2], b1[3], 0x0c0c0501u);
-        dg[t][2][c] = gather(b0[0], b0[1], b0[2], b0[3], 0x0c0c0400u);
-      }
-    }
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));      // over the four k quarters: row j's largest |x'| in this wave's k range
+      // A NaN or an infinity among row j's scaled activations has no digits.  The reference's GEMM returns NaN or an
+      // infinity in every output of that activation row; here this wave's share of them, and so their sum, is NaN.
+      const int bad = (__ballot(!finite) >> j & 0x0001000100010001ull) != 0 ? 1 : 0;
+      mx = bad ? 1.0f : mx;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) ur[r] = __shfl(unit, 4 * q + r) * s_one;
+      for (int r = 0; r < 4; ++r) poison[mt][r] = __shfl(bad, 4 * q + r) != 0;
+      int e = 0;
+      (void)frexpf(mx, &e);                     // mx = f * 2^e, f in [0.5, 1)
+      const float unit = mx > 0.0f ? ldexpf(1.0f, e - 5) : 1.0f;    // |x'| / unit < 32
+      const float inv16 = 65536.0f / unit;      // exact: a power of two
+      // second pass: n = round(x' / unit * 2^16) sits in the low mantissa bits of b = x' * inv16 + 1.5 * 2^23
+      // (|n| <= 2^21), and n = 2^16 d0 + 2^8 d1 + d2 with d1, d2 in [-128, 127]: d2 is byte 0 of b, d1 byte 1 of
+      // b + 0x80, d0 byte 2 of b + 0x8080 less the 0x40 that the constant leaves there (adding 0xC00000 removes it).
+#pragma unroll
+      for (int t = 0; t < kSteps; ++t) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          uint32_t b0[4], b1[4], b2[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            b0[i] = __builtin_bit_cast(uint32_t, __builtin_fmaf(xp[t][4 * c + i], inv16, 12582912.0f));
+            b1[i] = b0[i] + 0x80u;
+            b2[i] = b0[i] + 0xC08080u;
+          }
+          dg[mt][t][0][c] = gather(b2[0], b2[1], b2[2], b2[3], 0x0c0c0602u);
+          dg[mt][t][1][c] = gather(b1[0], b1[1], b1[2], b1[3], 0x0c0c0501u);
+          dg[mt][t][2][c] = gather(b0[0], b0[1], b0[2], b0[3], 0x0c0c0400u);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) ur[mt][r] = __shfl(unit, 4 * q + r) * s_one;
+    }
   }
 
   // The waves run freely through RBB blocks of 16 rows (no barrier in between, so one wave's
@@ -376,17 +409,20 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
   for (int seg0 = 0; seg0 < nrb; seg0 += kSegBlocks) {
     const int seg_end = seg0 + kSegBlocks < nrb ? seg0 + kSegBlocks : nrb;
     for (int base = seg0; base < seg_end; base += RBB) {
-      floatx4_t tot[RBB];
+      floatx4_t tot[RBB][MT];
 #pragma unroll
       for (int u = 0; u < RBB; ++u) {
         const int d = u % D;
         const int rb = base + u;
-        tot[u] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        if (rb < nrb) {          // same for every thread of the workgroup
 #pragma unroll
-          for (int g = 0; g < GPW; ++g) {
-            if constexpr (kInt4) {
-              floatx4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int mt = 0; mt < MT; ++mt) tot[u][mt] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        if (rb < nrb) {          // same for every thread of the workgroup
+          if constexpr (kInt4) {
+#pragma unroll
+            for (int g = 0; g < GPW; ++g) {
+              floatx4_t acc[MT];
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
               for (int t = 0; t < 4; ++t) {
                 // one xor turns the eight two's-complement nibbles into code + 8; every pair of
@@ -398,49 +434,68 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
                 c4[1] = and_or(p >> 4, 0x000F000Fu, kBase);
                 c4[2] = and_or(p >> 8, 0x000F000Fu, kBase);
                 c4[3] = and_or(p >> 12, 0x000F000Fu, kBase);
-                acc = Mfma16<CT>::run(xa[g][t], *reinterpret_cast<const vec_t *>(&c4), acc);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                  acc[mt] = Mfma16<CT>::run(xa[mt][g][t], *reinterpret_cast<const vec_t *>(&c4), acc[mt]);
               }
               const float sr = to_f32(sc[d][g]);
 #pragma unroll
-              for (int r = 0; r < 4; ++r) tot[u][r] = __builtin_fmaf(sr, acc[r] - cor[g][r], tot[u][r]);
+              for (int mt = 0; mt < MT; ++mt) {
+                if constexpr (MT == 1) {
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) tot[u][mt][r] = __builtin_fmaf(sr, acc[mt][r] - cor[g][r], tot[u][mt][r]);
+                } else {
+                  const floatx4_t cr = *reinterpret_cast<const floatx4_t *>(corbuf + (mt * GPW + g) * (kMbWaves * 16) + 4 * q);
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) tot[u][mt][r] = __builtin_fmaf(sr, acc[mt][r] - cr[r], tot[u][mt][r]);
+                }
+              }
             }
-          }
-          if constexpr (!kInt4) {
-            i32x4_t s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0}, s2 = {0, 0, 0, 0};
+          } else {
+            i32x4_t s0[MT], s1[MT], s2[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) s0[mt] = s1[mt] = s2[mt] = i32x4_t{0, 0, 0, 0};
 #pragma unroll
             for (int t = 0; t < kSteps; ++t) {
               const i32x4_t bw = __builtin_bit_cast(i32x4_t, w[d][t]);
-              s0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[t][0], bw, s0, 0, 0, 0);
-              s1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[t][1], bw, s1, 0, 0, 0);
-              s2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[t][2], bw, s2, 0, 0, 0);
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt) {
+                s0[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[mt][t][0], bw, s0[mt], 0, 0, 0);
+                s1[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[mt][t][1], bw, s1[mt], 0, 0, 0);
+                s2[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(dg[mt][t][2], bw, s2[mt], 0, 0, 0);
+              }
             }
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              float v = static_cast<float>(s0[r]);
-              v = __builtin_fmaf(static_cast<float>(s1[r]), 1.0f / 256.0f, v);
-              v = __builtin_fmaf(static_cast<float>(s2[r]), 1.0f / 65536.0f, v);
-              tot[u][r] = poison[r] ? __builtin_nanf("") : v * ur[r];
-            }
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                float v = static_cast<float>(s0[mt][r]);
+                v = __builtin_fmaf(static_cast<float>(s1[mt][r]), 1.0f / 256.0f, v);
+                v = __builtin_fmaf(static_cast<float>(s2[mt][r]), 1.0f / 65536.0f, v);
+                tot[u][mt][r] = poison[mt][r] ? __builtin_nanf("") : v * ur[mt][r];
+              }
           }
         }
         issue(d, rb + D);      // into the registers just consumed; the other block of the ring stays in flight
       }
 
-      // tot[u][r] = this wave's share of Y[activation row 4q+r][weight row j of block base+u]
+      // tot[u][mt][r] = this wave's share of Y[activation row 16 mt + 4q + r][weight row j of block base+u]
 #pragma unroll
       for (int u = 0; u < RBB; ++u)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) partial[((u * kMbWaves + wave) * 4 + r) * 64 + lane] = tot[u][r];
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) partial[(((u * MT + mt) * kMbWaves + wave) * 4 + r) * 64 + lane] = tot[u][mt][r];
       __syncthreads();
-      if (threadIdx.x < RBB * 256) {
-        const int u = threadIdx.x >> 8;
-        const int r = (threadIdx.x >> 6) & 3;
-        const int l = threadIdx.x & 63;
+      for (int idx = threadIdx.x; idx < RBB * MT * 256; idx += kMbThreads) {
+        const int um = idx >> 8;             // u * MT + mt
+        const int r = (idx >> 6) & 3;
+        const int l = idx & 63;
         float v = 0.0f;
 #pragma unroll
-        for (int wv = 0; wv < kMbWaves; ++wv) v += partial[((u * kMbWaves + wv) * 4 + r) * 64 + l];
-        const int m = 4 * (l >> 4) + r;
-        ybuf[m * kSegRows + (base - seg0 + u) * 16 + (l & 15)] = v;
+        for (int wv = 0; wv < kMbWaves; ++wv) v += partial[((um * kMbWaves + wv) * 4 + r) * 64 + l];
+        const int m = 16 * (um % MT) + 4 * (l >> 4) + r;
+        ybuf[m * kSegRows + (base - seg0 + um / MT) * 16 + (l & 15)] = v;
       }
       __syncthreads();            // the next round overwrites the partial tiles; the flush reads ybuf
     }
@@ -458,10 +513,10 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
   }
 }
 
-template <typename CT, typename XT, bool kInt4, int GPW, bool kF32 = false>
+template <typename CT, typename XT, bool kInt4, int GPW, bool kF32 = false, int MT = 1>
 __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
 {
-  mblock_body<CT, XT, kInt4, GPW, kF32>(a, a.wq, a.scales, a.x, a.y, a.M, blockIdx.y);
+  mblock_body<CT, XT, kInt4, GPW, kF32, MT>(a, a.wq, a.scales, a.x, a.y, a.M, blockIdx.y);
 }
 
 // Token-sorted expert segments with few rows each (MoE decode): blockIdx.y is the expert, whose weight is streamed
@@ -500,15 +555,27 @@ int64_t gcd64(int64_t x, int64_t y)
   return x;
 }
 
-template <typename CT, typename XT, bool kInt4>
+// groups per wave that a kernel with MT tiles is built for: the operands of 32 rows (bf16 values or int8 digit
+// planes) fit the 128 registers at one group per wave; with two, the int4 kernel spills 28-35 registers in its main loop
+constexpr int mb_max_gpw(bool /*int4*/, int mt) { return mt == 1 ? 2 : 1; }
+
+template <typename CT, typename XT, bool kInt4, bool kF32 = false>
 int launch_gpw(const MbArgs &m, size_t lds, hipStream_t s)
 {
   const dim3 grid(static_cast<unsigned>(m.blocks_per_class * m.V),
                   static_cast<unsigned>((m.groups + m.slice_groups - 1) / m.slice_groups));
   const int gpw = (m.slice_groups + kMbWaves - 1) / kMbWaves;
-  if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 1>), grid, dim3(kMbThreads), lds, s, m);
-  else if (gpw <= 2) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 2>), grid, dim3(kMbThreads), lds, s, m);
-  else return CAIFX_ERR_UNSUPPORTED;
+  if (m.M <= 16) {
+    if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 1, kF32>), grid, dim3(kMbThreads), lds, s, m);
+    else if (gpw <= 2) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 2, kF32>), grid, dim3(kMbThreads), lds, s, m);
+    else return CAIFX_ERR_UNSUPPORTED;
+  } else {
+    if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 1, kF32, 2>), grid, dim3(kMbThreads), lds, s, m);
+    else if constexpr (mb_max_gpw(kInt4, 2) >= 2) {
+      if (gpw <= 2) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 2, kF32, 2>), grid, dim3(kMbThreads), lds, s, m);
+      else return CAIFX_ERR_UNSUPPORTED;
+    } else return CAIFX_ERR_UNSUPPORTED;
+  }
   return launch_status();
 }
 
@@ -536,13 +603,7 @@ int launch_grouped_xt(const MbArgs &m, const MbGroup &g, int experts, int x_dtyp
 template <typename XT>
 int launch_f32(const MbArgs &m, size_t lds, hipStream_t s)
 {
-  const dim3 grid(static_cast<unsigned>(m.blocks_per_class * m.V),
-                  static_cast<unsigned>((m.groups + m.slice_groups - 1) / m.slice_groups));
-  const int gpw = (m.slice_groups + kMbWaves - 1) / kMbWaves;
-  if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<bf16_t, XT, false, 1, true>), grid, dim3(kMbThreads), lds, s, m);
-  else if (gpw <= 2) hipLaunchKernelGGL((mblock_kernel<bf16_t, XT, false, 2, true>), grid, dim3(kMbThreads), lds, s, m);
-  else return CAIFX_ERR_UNSUPPORTED;
-  return launch_status();
+  return launch_gpw<bf16_t, XT, false, true>(m, lds, s);
 }
 
 template <typename CT>
@@ -568,27 +629,70 @@ int compute_units()
 
 }  // namespace
 
-constexpr int64_t kMbSliceK = kMbWaves * 2 * 128;      // reduction length one workgroup covers
+constexpr int kMbMaxRows = 32;                          // two tiles of 16 activation rows
+constexpr int64_t kMbMaxSlices = 64;
+
+// longest reduction one workgroup covers: 16 waves times the groups a wave can hold operands for
+static int64_t mb_reach(int64_t M) { return kMbWaves * 128 * mb_max_gpw(false, M > 16 ? 2 : 1); }
+
+// Reduction length per workgroup the launch is planned with.  The int8 prologue (scaled activations cut into digit
+// planes) costs a workgroup time in proportion to its k range, while its share of the weight shrinks with N: at
+// K = 4096, 16 rows, half the reach plus the pass that adds the two slices measured 17.6 -> 12.5 us (fp32 compute,
+// N = 4096), 26.1 -> 21.9 us (fp32, N = 14336), 13.5 -> 11.7 us (bf16, N = 4096), 18.7 -> 18.9 us (bf16, N = 14336).
+// int4 has no such prologue and loses (9.3 -> 9.0 us at N = 4096 but 14.4 -> 15.2 us at N = 14336).
+static int64_t mb_slice_k(const GemmArgs &g)
+{
+  const int64_t reach = mb_reach(g.M);
+  if (g.M > 16 || g.w.kind == CAIFX_W_INT4_GROUP) return reach;
+  const int64_t n_max = g.compute_dtype == CAIFX_F32 ? 32768 : 8192;
+  return g.N <= n_max ? reach / 2 : reach;
+}
+
+static size_t mb_lds_bytes(bool int4, int mt, int slice_groups)
+{
+  size_t floats = static_cast<size_t>(mb_reduce_blocks(int4, mt)) * mt * kPartialFloats + static_cast<size_t>(16) * mt * kSegRows;
+  if (!int4) floats += static_cast<size_t>(slice_groups) * 128;      // staged scales (ones without a scale vector)
+  else if (mt > 1) floats += static_cast<size_t>(mt) * mb_max_gpw(true, mt) * kMbWaves * 16;      // group-sum corrections
+  return floats * sizeof(float);
+}
 
 size_t mblock_workspace_bytes(const GemmArgs &g)
 {
-  if (g.offsets || g.M < 1 || g.M > 16 || g.K <= kMbSliceK || g.K % 128 != 0 || g.K > 64 * kMbSliceK) return 0;
-  if (g.compute_dtype == CAIFX_F32 && g.w.kind == CAIFX_W_INT4_GROUP) return 0;
-  const int64_t slices = (g.K + kMbSliceK - 1) / kMbSliceK;
+  if (g.offsets || g.M < 1 || g.M > kMbMaxRows || g.K % 128 != 0) return 0;
+  const bool int4 = g.w.kind == CAIFX_W_INT4_GROUP;
+  if (g.compute_dtype == CAIFX_F32 && int4) return 0;
+  int64_t reach = mb_slice_k(g);
+  int64_t slices = (g.K + reach - 1) / reach;
+  if (slices > kMbMaxSlices) {
+    reach = mb_reach(g.M);
+    slices = (g.K + reach - 1) / reach;
+  }
+  if (slices < 2 || slices > kMbMaxSlices) return 0;
   return static_cast<size_t>(slices) * static_cast<size_t>(g.M) * static_cast<size_t>(g.N) * sizeof(float);
 }
 
 int mblock_forward(const GemmArgs &g, hipStream_t s)
 {
-  if (g.offsets || g.M < 1 || g.M > 16) return CAIFX_ERR_UNSUPPORTED;
-  if (g.N < 16 || g.N > (int64_t{1} << 30) || g.K % 128 != 0 || g.K > 64 * kMbSliceK) return CAIFX_ERR_UNSUPPORTED;
+  if (g.offsets || g.M < 1 || g.M > kMbMaxRows) return CAIFX_ERR_UNSUPPORTED;
+  if (g.N < 16 || g.N > (int64_t{1} << 30) || g.K % 128 != 0) return CAIFX_ERR_UNSUPPORTED;
   if (!aligned_to(g.w.q, 16) || !aligned_to(g.x, 16)) return CAIFX_ERR_UNSUPPORTED;
   const bool int4 = g.w.kind == CAIFX_W_INT4_GROUP;
   if (g.compute_dtype == CAIFX_F32 && int4) return CAIFX_ERR_UNSUPPORTED;
   // a reduction longer than one workgroup's reach is cut into slices whose sums meet in the caller's workspace
-  const int64_t slices = (g.K + kMbSliceK - 1) / kMbSliceK;
-  if (slices > 1 && (!g.workspace || g.workspace_bytes < mblock_workspace_bytes(g) || !aligned_to(g.workspace, 4)))
-    return CAIFX_ERR_UNSUPPORTED;
+  // (a shorter slice than the workgroup's reach is a choice: without room for its sums the full reach is used)
+  const int mt = g.M > 16 ? 2 : 1;
+  int64_t reach = mb_slice_k(g);
+  int64_t slices = (g.K + reach - 1) / reach;
+  const bool room = g.workspace && aligned_to(g.workspace, 4) &&
+                    g.workspace_bytes / sizeof(float) / static_cast<size_t>(g.M) / static_cast<size_t>(g.N) >= static_cast<size_t>(slices);
+  if (slices > kMbMaxSlices || (slices > 1 && !room)) {
+    reach = mb_reach(g.M);
+    slices = (g.K + reach - 1) / reach;
+    if (slices > kMbMaxSlices) return CAIFX_ERR_UNSUPPORTED;
+    if (slices > 1 && (!g.workspace || !aligned_to(g.workspace, 4) ||
+                       g.workspace_bytes < static_cast<size_t>(slices) * static_cast<size_t>(g.M) * static_cast<size_t>(g.N) * sizeof(float)))
+      return CAIFX_ERR_UNSUPPORTED;
+  }
 
   MbArgs m{};
   m.wq = static_cast<const uint8_t *>(g.w.q);
@@ -600,10 +704,10 @@ int mblock_forward(const GemmArgs &g, hipStream_t s)
   m.N = g.N;
   m.K = g.K;
   m.groups = static_cast<int>(g.K / 128);
-  m.slice_groups = slices > 1 ? static_cast<int>(kMbSliceK / 128) : m.groups;
+  m.slice_groups = static_cast<int>((m.groups + slices - 1) / slices);      // slices of equal length, the last may be shorter
+  slices = (m.groups + m.slice_groups - 1) / m.slice_groups;
   m.partial = slices > 1 ? static_cast<float *>(g.workspace) : nullptr;
   m.V = 1;
-  size_t lds = ((int4 ? 4 : 2) * kPartialFloats + 16 * kSegRows) * sizeof(float);      // RBB buffers of partial tiles + output staging
   if (int4) {
     const int gs = g.w.group_size;
     if (!g.w.scales || gs < 128 || (gs & (gs - 1)) != 0) return CAIFX_ERR_UNSUPPORTED;
@@ -617,7 +721,7 @@ int mblock_forward(const GemmArgs &g, hipStream_t s)
     m.scale_step = static_cast<int>(kMbThreads % P);
     m.V = static_cast<int>(V);
   }
-  if (!int4) lds += static_cast<size_t>(m.slice_groups) * 128 * sizeof(float);      // staged scales (ones without a scale vector)
+  const size_t lds = mb_lds_bytes(int4, mt, m.slice_groups);
   // one workgroup per compute unit over all slices: the prologue (the slice of X as operands, for int8 its digit
   // planes) is paid per workgroup, so each should own as many rows as the chip allows
   int target = static_cast<int>((compute_units() + slices - 1) / slices);
@@ -645,7 +749,7 @@ int mblock_grouped_forward(const GemmArgs &g, hipStream_t s)
   // worth it while a segment takes one or two passes of 16 rows; the tiled kernel streams an expert's weight
   // once per 128 rows
   if (g.M > 16 * static_cast<int64_t>(g.num_experts)) return CAIFX_ERR_UNSUPPORTED;
-  if (g.N < 16 || g.N > (int64_t{1} << 30) || g.K % 128 != 0 || g.K > kMbSliceK || !aligned_to(g.x, 16)) return CAIFX_ERR_UNSUPPORTED;
+  if (g.N < 16 || g.N > (int64_t{1} << 30) || g.K % 128 != 0 || g.K > mb_reach(16) || !aligned_to(g.x, 16)) return CAIFX_ERR_UNSUPPORTED;
   const bool int4 = g.w.kind == CAIFX_W_INT4_GROUP;
   MbArgs m{};
   m.x = g.x;
@@ -657,7 +761,6 @@ int mblock_grouped_forward(const GemmArgs &g, hipStream_t s)
   m.groups = static_cast<int>(g.K / 128);
   m.slice_groups = m.groups;
   m.V = 1;
-  size_t lds = ((int4 ? 4 : 2) * kPartialFloats + 16 * kSegRows) * sizeof(float);
   if (int4) {
     const int gs = g.w.group_size;
     if (!g.scales_ptrs || gs < 128 || (gs & (gs - 1)) != 0) return CAIFX_ERR_UNSUPPORTED;
@@ -671,7 +774,7 @@ int mblock_grouped_forward(const GemmArgs &g, hipStream_t s)
     m.scale_step = static_cast<int>(kMbThreads % P);
     m.V = static_cast<int>(V);
   }
-  if (!int4) lds += static_cast<size_t>(g.K) * sizeof(float);
+  const size_t lds = mb_lds_bytes(int4, 1, m.groups);
   const int64_t nrb_class = ((g.N + m.V - 1) / m.V + 15) / 16;
   int64_t bpc = 2 * static_cast<int64_t>(compute_units()) / (static_cast<int64_t>(g.num_experts) * m.V);
   if (bpc < 1) bpc = 1;

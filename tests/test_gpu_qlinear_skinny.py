@@ -172,10 +172,39 @@ def test_one_hot_reads_a_weight_column_exactly(orc):
 @pytest.mark.parametrize("kind", ["int4", "int8pc", "int8pt"])
 @pytest.mark.parametrize("M", [17, 24, 32])
 def test_two_row_blocks_of_the_decode_kernel(orc, kind, M):
-    # 17..32 rows run as two launches of the 16-row kernel (same accuracy class as M <= 16); row 16 onwards
-    # must come out of the second launch with the right offsets into X and Y
+    # 17..32 rows: two tiles of 16 activation rows share one pass over the weight (same accuracy class as
+    # M <= 16); a workgroup then reaches 2048 of the reduction, so K = 1024 is one slice, K = 4096 two and
+    # K = 5120 three with a short last one, meeting in the workspace.  Rows 16 onwards are the second tile.
     _check(orc, np.random.default_rng(700 + M), M, 1536, 1024, kind, 2, 2)
     _check(orc, np.random.default_rng(701 + M), M, 200, 4096, kind, 1, 1, yd=2)
+    _check(orc, np.random.default_rng(702 + M), M, 1792, 4096, kind, 2, 0)
+    _check(orc, np.random.default_rng(703 + M), M, 272, 5120, kind, 2, 2, yd=1)
+
+
+@pytest.mark.parametrize("kind", ["int4", "int8pc"])
+def test_two_row_blocks_without_a_workspace_run_16_rows_at_a_time(orc, kind):
+    # without room for the slices' partial sums the same rows go through two launches of the 16-row form;
+    # both forms are of one accuracy class and agree to fp32 summation order
+    rng = np.random.default_rng(12)
+    N, K, M = 528, 4096, 27
+    ow, dw = make_weight(orc, rng, N, K, kind)
+    xt = dev_as(rng.normal(0, 1, (M, K)), 2)
+    want = orc.frozen_linear_forward(host(xt), ow, 2)
+    import torch
+    none = torch.empty(0, dtype=torch.uint8, device="cuda")
+    y0 = host(T.qlinear_forward(xt, dw, 2, 0, workspace=none))
+    y1 = host(T.qlinear_forward(xt, dw, 2, 0))
+    assert max_rel_err(y0, want) <= TIGHT_POST
+    assert max_rel_err(y1, want) <= TIGHT_POST
+    assert np.abs(y0 - y1).max() <= 2e-4 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("M", [17, 32])
+@pytest.mark.parametrize("xd", [0, 2])
+def test_two_row_blocks_fp32_compute(orc, M, xd):
+    # fp32 compute type with int8 codes: digit planes of the unrounded activations, 1e-4 contract
+    _check(orc, np.random.default_rng(750 + M + xd), M, 1024, 4096, "int8pc", 0, xd)
+    _check(orc, np.random.default_rng(751 + M + xd), M, 336, 1152, "int8pt", 0, xd)
 
 
 @pytest.mark.parametrize("cd,xd", [(2, 0), (2, 1), (1, 0), (1, 2)])
@@ -200,7 +229,7 @@ def test_one_row_int8_casts_the_activations_to_the_compute_dtype(orc, kind, K, c
 
 
 @pytest.mark.parametrize("kind", ["int8pc", "int8pt", "int4"])
-@pytest.mark.parametrize("M", [1, 2, 4, 16, 24])
+@pytest.mark.parametrize("M", [1, 2, 4, 16, 24, 32])
 def test_non_finite_activations_are_not_masked(orc, kind, M):
     # A NaN or an infinity in an activation row reaches every output of that row in the reference (dequantise +
     # GEMM: every output multiplies every activation, and 0 * inf is NaN too).  The integer-matrix-core kernels
@@ -225,7 +254,7 @@ def test_non_finite_activations_are_not_masked(orc, kind, M):
 
 
 @pytest.mark.parametrize("kind", ["int4", "int8pc"])
-@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("M", [1, 4, 16, 32])
 def test_post_scaled_kernels_on_correlated_inputs(orc, kind, M):
     # The memory-bound kernels skip the reference's rounding of code*scale to bf16.  On N(0,1) activations those
     # rounding differences add up like a random walk (about 2e-3 of max|ref|).  Correlated inputs are the worst

@@ -53,11 +53,11 @@ def test_two_calls_second_smaller_match_the_workspace_form(orc, kind, cd, xd):
 
 @pytest.mark.parametrize("kind", ["int4", "int8pc"])
 def test_long_reduction_slices_meet_in_the_static_buffer(orc, kind):
-    # K > 4096 with up to 32 rows: the 16-row decode kernel's slices of the reduction use the same buffer
+    # K > 4096 with up to 16 rows, K > 2048 with 17..32: the decode kernel's slices of the reduction use the same buffer
     rng = np.random.default_rng(47)
     N, K = 1024, 8192
     ow, dw = make_weight(orc, rng, N, K, kind)
-    for M in (16, 24, 5):
+    for M in (16, 24, 5, 32):
         assert 0 < _need(M, dw, 2, 2) <= SCRATCH_BYTES
         x = dev_as(rng.normal(0, 1, (M, K)), 2)
         st, y = _static(x, dw, 2)
