@@ -238,7 +238,7 @@ def decode_other_rows(torch, T, dev, gen, capture, time_graph):
     `decode_down_proj`: the FFN down projection of the same model (N = 4096, K = 14336), M = 1 and 16."""
     out = {"decode_tall_M1": {}, "decode_down_proj": {}}
     x1 = torch.empty(1, K_DEC, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16)
-    ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    ws = torch.empty(4 << 20, dtype=torch.uint8, device=dev)      # the 16-row kernel's reduction slices at K = 14336: 1.8 MB
     N_TALL = 8 * N_DEC
     w = torch.empty(N_TALL, K_DEC, device=dev).normal_(0, 0.02, generator=gen)
     p4, s4 = T.quantize_int4_per_group(w, 128)
@@ -432,9 +432,12 @@ def fp32_rows(torch, T, dev, gen, capture, time_graph):
     q, s = T.quantize_int8(w, per_channel=True)
     del w
     fw = T.FrozenWeight(q.reshape(-1), T.W_INT8, s, N, K, N)
-    ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    from caif_amd import capi
     rows = {}
     for M, L in ((16, 32), (2048, 8)):
+        # the workspace the library asks for (few rows: partial sums of reduction slices / row ranges)
+        nb = max(capi.lib().caifx_qlinear_workspace_bytes(M, N, K, T.F32, T.F32, T.W_INT8, b) for b in (0, 1))
+        ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=dev)
         x = torch.empty(M, K, device=dev).normal_(0, 1, generator=gen)
         dy = torch.empty(M, N, device=dev).normal_(0, 1e-3, generator=gen)
         y, dx = torch.empty(M, N, device=dev), torch.empty(M, K, device=dev)

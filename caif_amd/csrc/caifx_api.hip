@@ -113,10 +113,8 @@ size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtyp
   a.w.kind = w_kind;
   const size_t f32_bytes = mfma_f32_workspace_bytes(a, backward != 0);
   size_t bytes = mfma_workspace_bytes(a, backward != 0);
-  if (!backward) {
-    const size_t decode_bytes = mblock_workspace_bytes(a);
-    if (decode_bytes > bytes) bytes = decode_bytes;
-  }
+  const size_t decode_bytes = backward ? dxrows_workspace_bytes(a) : mblock_workspace_bytes(a);
+  if (decode_bytes > bytes) bytes = decode_bytes;
   return f32_bytes > bytes ? f32_bytes : bytes;
 }
 
@@ -248,6 +246,12 @@ static int backward_impl(int64_t M, int64_t N, int64_t K, const void *dy, int dy
   GemmArgs a = make_args(M, N, K, dy, dy_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size,
                          dx, dx_dtype, workspace, workspace_bytes);
   hipStream_t s = as_stream(stream);
+  // up to 16 rows of int8 codes whose scales do not depend on the weight row: one pass over the weight at the
+  // memory rate, whatever the compute type
+  if (M <= 16 && w_kind == CAIFX_W_INT8) {
+    st = dxrows_backward(a, s);
+    if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, dx, dx_dtype, M * K, stream);
+  }
   if (compute_dtype == CAIFX_F32 || float_kind(w_kind)) {
     st = mfma_f32_backward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, dx, dx_dtype, M * K, stream);

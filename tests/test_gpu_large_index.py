@@ -53,13 +53,16 @@ def test_flat_indices_beyond_2_31(kind):
         dy = torch.zeros(M, N, device="cuda", dtype=torch.bfloat16)
         dy[:, -R:] = torch.randn(M, R, device="cuda", generator=gen).to(torch.bfloat16)
         dx = T.qlinear_backward_input(dy, fw, T.BF16)
-        assert _rel(dx, dy[:, -R:].float() @ w_bf16) <= 2e-5, (kind, M)
+        # up to 16 rows of int8 codes take the few-row kernel, which skips the bf16 rounding of code*scale as well
+        tol = 4e-3 if (M <= 16 and kind == "int8pt") else 2e-5
+        assert _rel(dx, dy[:, -R:].float() @ w_bf16) <= tol, (kind, M)
     # fp32 compute type on the same weight
     x = torch.randn(16, K, device="cuda", generator=gen)
     assert _rel(T.qlinear_forward(x, fw, T.F32)[:, -R:], x @ dense_top.t()) <= 1e-4, kind
-    dy = torch.zeros(40, N, device="cuda")
-    dy[:, -R:] = torch.randn(40, R, device="cuda", generator=gen)
-    assert _rel(T.qlinear_backward_input(dy, fw, T.F32), dy[:, -R:] @ dense_top) <= 1e-4, kind
+    for M in (16, 40):                                              # few-row kernel, tiled kernel
+        dy = torch.zeros(M, N, device="cuda")
+        dy[:, -R:] = torch.randn(M, R, device="cuda", generator=gen)
+        assert _rel(T.qlinear_backward_input(dy, fw, T.F32), dy[:, -R:] @ dense_top) <= 1e-4, (kind, M)
 
 
 def test_quantisers_beyond_2_31_elements():

@@ -289,3 +289,84 @@ def test_post_scaled_kernels_on_correlated_inputs(orc, kind, M):
     worst = max(cases.values())
     print(f"post-scaled {kind} M={M}: " + ", ".join(f"{w}/{x}={e:.2e}" for (w, x), e in cases.items()))
     assert worst <= TOL_16, cases
+
+
+# ---------------------------------------------------------------- input gradient for a few rows
+
+def _check_dx(orc, rng, M, N, K, kind, cd, xd, yd=0, workspace=None):
+    ow, dw = make_weight(orc, rng, N, K, kind)
+    dy = dev_as(rng.normal(0, 1e-3, (M, N)).astype(np.float32), xd)
+    dx = host(T.qlinear_backward_input(dy, dw, cd, yd, workspace=workspace))
+    want = orc.frozen_linear_backward(host(dy), ow, cd)
+    if yd != 0:
+        want = orc.round_to_dtype(want, yd)
+    err = max_rel_err(dx, want)
+    assert err <= (TOL_32 if cd == 0 else TOL_16), (M, N, K, kind, cd, xd, err)
+    return err
+
+
+@pytest.mark.parametrize("kind", ["int8pc", "int8pt", "int8raw"])
+@pytest.mark.parametrize("M", [1, 5, 16])
+def test_input_gradient_few_rows_fp32(orc, kind, M):
+    # dX = dY W for up to 16 rows of int8 codes streams the weight once through the fp32 matrix core when the scale
+    # of W[n][k] does not depend on n (square per-channel weight: K mod N = 0; one scale; none).  Shapes: BASELINE
+    # config 1 (4096 x 4096), a row count that is no multiple of a wave's 16 rows (N = 1000), a single column slab
+    # (K = 128), fewer rows than one workgroup pass (N = 40).
+    rng = np.random.default_rng(300 + M)
+    for N, K in ((4096, 4096), (1000, 1024), (3000, 128), (40, 256)):
+        if kind == "int8pc" and K % N != 0:
+            continue
+        assert _check_dx(orc, rng, M, N, K, kind, 0, 0) <= 2e-6, (N, K)
+
+
+@pytest.mark.parametrize("cd,xd,yd", [(2, 2, 0), (2, 0, 2), (1, 1, 1), (1, 0, 0), (0, 2, 0), (0, 1, 2)])
+def test_input_gradient_few_rows_dtype_mixes(orc, cd, xd, yd):
+    # 16-bit compute types: dY is rounded to the compute type first (the layer's cast of its input); the weight is
+    # not (post-scaled class, like the decode forward)
+    rng = np.random.default_rng(cd * 9 + xd * 3 + yd)
+    for kind, N, K in (("int8pc", 512, 1024), ("int8pt", 777, 384)):
+        err = _check_dx(orc, rng, 7, N, K, kind, cd, xd, yd)
+        if cd != 0 and yd == 0:
+            assert err <= TIGHT_POST
+
+
+def test_input_gradient_few_rows_other_paths(orc):
+    # per-channel scales whose index depends on the weight row (K mod N != 0), int4 codes, more than 16 rows and a
+    # call without a workspace go to the tiled kernels; all must agree with the oracle
+    import torch
+    rng = np.random.default_rng(31)
+    _check_dx(orc, rng, 8, 1536, 1024, "int8pc", 0, 0)
+    _check_dx(orc, rng, 8, 512, 1024, "int4", 2, 2)
+    _check_dx(orc, rng, 17, 512, 512, "int8pc", 0, 0)
+    none = torch.empty(0, dtype=torch.uint8, device="cuda")
+    _check_dx(orc, rng, 16, 2048, 2048, "int8pc", 0, 0, workspace=none)
+    _check_dx(orc, rng, 3, 40, 128, "int8pt", 0, 0, workspace=none)     # one workgroup: no workspace needed
+
+
+def test_input_gradient_few_rows_is_the_adjoint_of_the_forward(orc):
+    # <dY, X W^T> = <dY W, X> with both sides from the device kernels (fp32 compute)
+    rng = np.random.default_rng(32)
+    N, K, M = 1024, 1024, 16
+    ow, dw = make_weight(orc, rng, N, K, "int8pc")
+    x = dev_as(rng.normal(0, 1, (M, K)).astype(np.float32), 0)
+    dy = dev_as(rng.normal(0, 1, (M, N)).astype(np.float32), 0)
+    y = host(T.qlinear_forward(x, dw, 0)).astype(np.float64)
+    dx = host(T.qlinear_backward_input(dy, dw, 0)).astype(np.float64)
+    lhs = (host(dy).astype(np.float64) * y).sum()
+    rhs = (dx * host(x).astype(np.float64)).sum()
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), abs(rhs))
+
+
+def test_input_gradient_few_rows_keeps_non_finite_gradients_in_their_row(orc):
+    rng = np.random.default_rng(33)
+    N, K, M = 512, 512, 6
+    ow, dw = make_weight(orc, rng, N, K, "int8pt")
+    for bad in (np.nan, np.inf):
+        dy = rng.normal(0, 1e-3, (M, N)).astype(np.float32)
+        dy[2, 77] = bad
+        dx = host(T.qlinear_backward_input(dev_as(dy, 0), dw, 0))
+        want = orc.frozen_linear_backward(dy, ow, 0)
+        assert not np.isfinite(want[2]).any() and not np.isfinite(dx[2]).any()
+        assert np.array_equal(np.isfinite(dx), np.isfinite(want))
+        good = [m for m in range(M) if m != 2]
+        assert max_rel_err(dx[good], want[good]) <= TOL_32
