@@ -55,6 +55,12 @@ def test_decode_full_width_m1(orc, kind):
     _check(orc, np.random.default_rng(17), 1, 14336, 4096, kind, cd=2, xd=2)
 
 
+@pytest.mark.parametrize("kind", ["int4", "int8pc"])
+def test_decode_full_width_two_row_tiles(orc, kind):
+    # the decode geometry at its full width with 32 rows: two tiles, two reduction slices, 7 residue classes (int8)
+    _check(orc, np.random.default_rng(18), 32, 14336, 4096, kind, cd=2, xd=2)
+
+
 @pytest.mark.parametrize("kind", ["int4", "int8pc", "int8pt"])
 @pytest.mark.parametrize("N,K,M", [(4096, 14336, 1), (4096, 14336, 16), (1024, 8192, 4), (528, 11008, 9), (640, 4224, 24),
                                    (2048, 8192, 1), (1024, 11264, 1), (1536, 5120, 1), (512, 16384, 1), (1027, 9216, 1)])
