@@ -21,6 +21,11 @@ def test_replays_equal_eager_results():
     fw8 = T.FrozenWeight(q8.reshape(-1), T.W_INT8, s8, N, K, N)
     p4, s4 = T.quantize_int4_per_group(w.reshape(N, K), 128)
     fw4 = T.FrozenWeight(p4, T.W_INT4_GROUP, s4, N, K, 1, 128)
+    # K = 4096: the row-block decode kernel runs int8 in two reduction slices whose sums meet in the workspace
+    # (16 rows, 24 rows in two tiles, fp32 compute)
+    wk = torch.empty(4096, N, device=dev).normal_(0, 0.02, generator=gen)
+    q8k, s8k = T.quantize_int8(wk, per_channel=True)
+    fw8k = T.FrozenWeight(q8k.reshape(-1), T.W_INT8, s8k, N, 4096, N)
     experts = []
     for _ in range(E):
         we = torch.empty(D, D, device=dev).normal_(0, 0.02, generator=gen)
@@ -33,6 +38,8 @@ def test_replays_equal_eager_results():
     x1, x16, x64 = (torch.empty(m, K, device=dev, dtype=torch.bfloat16) for m in (1, 16, 64))
     dy64 = torch.empty(64, N, device=dev, dtype=torch.bfloat16)
     xf = torch.empty(16, K, device=dev)
+    x16k, x24k = (torch.empty(m, 4096, device=dev, dtype=torch.bfloat16) for m in (16, 24))
+    xfk = torch.empty(5, 4096, device=dev)
     tok = torch.empty(Tk, D, device=dev, dtype=torch.bfloat16)
     idx = torch.empty(Tk, top_k, device=dev, dtype=torch.int32)
     wts = torch.empty(Tk, top_k, device=dev, dtype=torch.bfloat16)
@@ -43,10 +50,11 @@ def test_replays_equal_eager_results():
         g = torch.Generator(device=dev)
         g.manual_seed(seed)
         wsrc.normal_(0, 0.02, generator=g)
-        for t in (x1, x16, x64, tok):
+        for t in (x1, x16, x64, tok, x16k, x24k):
             t.copy_(torch.empty(t.shape, device=dev).normal_(0, 1, generator=g))
         dy64.copy_(torch.empty(64, N, device=dev).normal_(0, 1e-2, generator=g))
         xf.normal_(0, 1, generator=g)
+        xfk.normal_(0, 1, generator=g)
         idx.copy_(torch.randint(0, E, (Tk, top_k), device=dev, generator=g).to(torch.int32))
         wts.copy_(torch.softmax(torch.empty(Tk, top_k, device=dev).normal_(0, 1, generator=g), dim=1))
 
@@ -61,6 +69,9 @@ def test_replays_equal_eager_results():
         out["y64"] = T.qlinear_forward(x64, fw4, T.BF16, workspace=ws)
         out["dx64"] = T.qlinear_backward_input(dy64, fw8, T.BF16, workspace=ws)
         out["yf"] = T.qlinear_forward(xf, fw8, T.F32, workspace=ws)
+        out["y16k"] = T.qlinear_forward(x16k, fw8k, T.BF16, workspace=ws)
+        out["y24k"] = T.qlinear_forward(x24k, fw8k, T.BF16, workspace=ws)
+        out["yfk"] = T.qlinear_forward(xfk, fw8k, T.F32, workspace=ws)
         dmap, offs = T.moe_build_dispatch_map(idx, E)                            # counters, scans
         packed = T.moe_dispatch(tok, idx, dmap, offs, rows, out=torch.empty(rows, D, device=dev, dtype=torch.bfloat16))
         ye = T.qlinear_grouped_forward(packed, offs, gw, T.BF16, T.BF16, workspace=ws,
