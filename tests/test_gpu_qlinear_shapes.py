@@ -80,3 +80,22 @@ def test_argument_errors():
     assert L.caifx_qlinear_forward(*args(kind=1, group=0)) == 1
     assert L.caifx_qlinear_forward(*args(x=x.data_ptr() + 2)) == 5   # misaligned fp32 pointer
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_seeded_random_shapes_cross_every_kernel_boundary(orc, seed):
+    # forward and input gradient on shapes drawn around the row counts, reduction lengths and widths at which the
+    # dispatcher changes kernels (1/2 rows row-streaming, 3..16 and 17..32 row blocks in one or more reduction slices,
+    # the few-row input gradient, tiled GEMM with and without a shared reduction, the shape-agnostic floor for K not a
+    # multiple of 64), with every weight kind and compute type
+    rng = np.random.default_rng(9000 + seed)
+    Ms = [1, 2, 3, 4, 8, 15, 16, 17, 24, 31, 32, 33, 48, 64, 100]
+    Ns = [16, 24, 40, 64, 200, 512, 777, 1000, 1536, 2050]
+    Ks = [64, 96, 128, 256, 384, 512, 1024, 1280, 2048, 2176, 4096, 4224, 5120]
+    for _ in range(8):
+        M, N, K = (int(rng.choice(v)) for v in (Ms, Ns, Ks))
+        kind = str(rng.choice(["int4", "int8pc", "int8pt", "int8raw"]))
+        cd = int(rng.choice([0, 1, 2]))
+        xd = int(rng.choice([0, cd]))            # the compute type or fp32 activations
+        group = int(rng.choice([32, 128])) if K % 128 == 0 else 32
+        _fwd_bwd(orc, rng, M, N, K, kind, cd, xd, group=group)
