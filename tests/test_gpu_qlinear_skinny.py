@@ -376,3 +376,25 @@ def test_input_gradient_few_rows_keeps_non_finite_gradients_in_their_row(orc):
         assert np.array_equal(np.isfinite(dx), np.isfinite(want))
         good = [m for m in range(M) if m != 2]
         assert max_rel_err(dx[good], want[good]) <= TOL_32
+
+
+@pytest.mark.parametrize("yd", [1, 2])
+def test_fused_add_on_the_few_row_paths_equals_the_two_launches(orc, yd):
+    # the LoRA composition base.To(T) + branch on the decode kernels (two row tiles forward, few-row input gradient):
+    # the fused entry points must give the bits of the plain call followed by the element-wise Add
+    import torch
+    rng = np.random.default_rng(60 + yd)
+    N, K = 512, 4096
+    ow, dw = make_weight(orc, rng, N, K, "int8pt")
+    x = dev_as(rng.normal(0, 1, (24, K)), 2)
+    add_y = dev_as(rng.normal(0, 1, (24, N)), yd)
+    fused = T.qlinear_forward(x, dw, 2, yd, addend=add_y)
+    plain = T.add(T.qlinear_forward(x, dw, 2, yd), add_y)
+    assert torch.equal(fused, plain)
+    dy = dev_as(rng.normal(0, 1e-2, (9, N)), 2)
+    add_x = dev_as(rng.normal(0, 1e-2, (9, K)), yd)
+    fused = T.qlinear_backward_input(dy, dw, 2, yd, addend=add_x)
+    plain = T.add(T.qlinear_backward_input(dy, dw, 2, yd), add_x)
+    assert torch.equal(fused, plain)
+    want = orc.round_to_dtype(orc.frozen_linear_backward(host(dy), ow, 2), yd) + host(add_x)
+    assert max_rel_err(host(fused), want) <= TOL_16
