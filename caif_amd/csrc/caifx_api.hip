@@ -246,9 +246,9 @@ static int backward_impl(int64_t M, int64_t N, int64_t K, const void *dy, int dy
   GemmArgs a = make_args(M, N, K, dy, dy_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size,
                          dx, dx_dtype, workspace, workspace_bytes);
   hipStream_t s = as_stream(stream);
-  // up to 16 rows of int8 codes whose scales do not depend on the weight row: one pass over the weight at the
-  // memory rate, whatever the compute type
-  if (M <= 16 && w_kind == CAIFX_W_INT8) {
+  // up to 16 rows of int8 codes whose scales do not depend on the weight row, or of int4 codes in groups of 128
+  // or more: one pass over the weight at the memory rate, whatever the compute type
+  if (M <= 16 && (w_kind == CAIFX_W_INT8 || w_kind == CAIFX_W_INT4_GROUP)) {
     st = dxrows_backward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, dx, dx_dtype, M * K, stream);
   }

@@ -10,6 +10,9 @@
 // few 1e-3 of the largest output for bf16, 1e-7 for the fp32 compute type).
 // That needs the scale of W[n][k] not to depend on n: scale index (n*K + k) mod period with K a multiple of the
 // period (which covers the per-output-channel scales of a square weight), one scale, or none.
+// Packed int4 codes in groups of 128 or more take the same route with the scale on the other operand: a slab of
+// 128 columns lies inside one group, so the scale of (row, group) multiplies the row's gradient before it enters
+// the A operand.
 //
 // A workgroup of 16 waves owns a slab of 128 columns (one cache line of every weight row it visits) and a range
 // of rows; the waves split the rows 16 at a time, add their 16 partial tiles through LDS in a fixed order and
@@ -31,20 +34,23 @@ constexpr int kDxWaveRows = 4 * kDxIter;     // rows a wave takes per pass
 constexpr int kDxPassRows = kDxWaves * kDxWaveRows;
 
 struct DxArgs {
-  const int8_t *wq;
-  const float *scales;
+  const int8_t *wq;         // int8 codes, or packed int4 (two codes per byte, even k in the low nibble)
+  const void *scales;       // int8: fp32 vector (see period); int4: fp16, one per row and group
   const void *dy;
   void *dx;
   int M;
   int y_dtype;
   int64_t N, K;
-  int period;              // 0: no scale, 1: scales[0], else scales[k % period]
+  int period;              // int8: 0: no scale, 1: scales[0], else scales[k % period]
+  int group_shift;         // int4: log2 of the group size (>= 7: a slab lies inside one group)
   int64_t rows_per_wg;     // rows of W per blockIdx.y
   float *partial;          // [gridDim.y][M][K] when the rows are split among workgroups, else null
 };
 
-// XT: type of dY in memory; CT: compute type dY is rounded to first, as the layer's cast of its input does
-template <typename XT, typename CT>
+// XT: type of dY in memory; CT: compute type dY is rounded to first, as the layer's cast of its input does.
+// kInt4: packed int4 codes; a lane's 8 codes are one dword, and the scale of (row, group) multiplies the row's
+// gradient on its way into the A operand (the slab's 128 columns share the group).
+template <typename XT, typename CT, bool kInt4>
 __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
 {
   extern __shared__ __attribute__((aligned(16))) float tiles[];      // [16 waves][8 codes][4][64], then [16][128] sums
@@ -56,7 +62,9 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
   const int64_t n_lo = static_cast<int64_t>(blockIdx.y) * a.rows_per_wg;
   const int64_t n_hi = n_lo + a.rows_per_wg < a.N ? n_lo + a.rows_per_wg : a.N;
   const XT *dy = static_cast<const XT *>(a.dy) + static_cast<int64_t>(j < a.M ? j : a.M - 1) * a.N;
-  const int8_t *wcol = a.wq + k0 + 8 * j;
+  const int8_t *wcol = a.wq + (kInt4 ? (k0 >> 1) + 4 * j : k0 + 8 * j);
+  const int64_t row_bytes = kInt4 ? a.K >> 1 : a.K;
+  const f16_t *s16 = static_cast<const f16_t *>(a.scales);
   const bool row_live = j < a.M;
 
   floatx4_t acc[8];
@@ -68,6 +76,7 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
   // number of loads in flight is known when the code is compiled and a stage is waited for without draining the
   // others.
   u32x2_t w[kDxStages][kDxIter];
+  f16_t ws[kDxStages][kDxIter];          // int4: scale of the row in this slab's group
   XT av[kDxStages][kDxIter];             // dY as loaded
   uint32_t keep[kDxStages][kDxIter];     // all ones where the row and the gradient row exist, else 0
   auto issue = [&](int st, int64_t base) {
@@ -75,7 +84,12 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
     for (int it = 0; it < kDxIter; ++it) {
       const int64_t n = base + 4 * it + q;
       const int64_t nn = n < n_hi ? n : n_hi - 1;          // rows past the range: a valid address, a zero gradient
-      w[st][it] = *reinterpret_cast<const u32x2_t *>(wcol + nn * a.K);
+      if constexpr (kInt4) {
+        w[st][it][0] = *reinterpret_cast<const uint32_t *>(wcol + nn * row_bytes);
+        ws[st][it] = s16[(nn * a.K + k0) >> a.group_shift];
+      } else {
+        w[st][it] = *reinterpret_cast<const u32x2_t *>(wcol + nn * row_bytes);
+      }
       av[st][it] = dy[nn];
       // (a mask on the bits, not a conditional expression: the compiler turns that into a load under a branch
       // with a full wait behind it)
@@ -85,10 +99,13 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
   auto multiply = [&](int st) {
 #pragma unroll
     for (int it = 0; it < kDxIter; ++it) {
-      const float g = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, round_through<CT>(to_f32<XT>(av[st][it]))) & keep[st][it]);
+      float g = round_through<CT>(to_f32<XT>(av[st][it]));
+      if constexpr (kInt4) g *= to_f32(ws[st][it]);
+      g = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, g) & keep[st][it]);
 #pragma unroll
       for (int b = 0; b < 8; ++b) {
-        const int code = static_cast<int>(w[st][it][b >> 2] << (24 - 8 * (b & 3))) >> 24;
+        const int code = kInt4 ? static_cast<int>(w[st][it][0] << (28 - 4 * b)) >> 28
+                               : static_cast<int>(w[st][it][b >> 2] << (24 - 8 * (b & 3))) >> 24;
         acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(g, static_cast<float>(code), acc[b], 0, 0, 0);
       }
     }
@@ -140,8 +157,11 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
     const int64_t k = k0 + (o & (kDxSlab - 1));
     if (m >= a.M) continue;
     float s = 1.0f;
-    if (a.period == 1) s = a.scales[0];
-    else if (a.period > 1) s = a.scales[k % a.period];
+    if constexpr (!kInt4) {
+      const float *s32 = static_cast<const float *>(a.scales);
+      if (a.period == 1) s = s32[0];
+      else if (a.period > 1) s = s32[k % a.period];
+    }
     const float v = tiles[o] * s;
     const int64_t at = static_cast<int64_t>(m) * a.K + k;
     if (a.partial) a.partial[static_cast<int64_t>(blockIdx.y) * a.M * a.K + at] = v;
@@ -159,28 +179,41 @@ int compute_units()
   return 256;
 }
 
-template <typename CT>
-int launch_ct(const DxArgs &a, int x_dtype, dim3 grid, size_t lds, hipStream_t s)
+template <typename CT, bool kInt4>
+int launch_xt(const DxArgs &a, int x_dtype, dim3 grid, size_t lds, hipStream_t s)
 {
-  if (x_dtype == CAIFX_F32) hipLaunchKernelGGL((dxrows_kernel<float, CT>), grid, dim3(kDxThreads), lds, s, a);
-  else if (x_dtype == CAIFX_BF16) hipLaunchKernelGGL((dxrows_kernel<bf16_t, CT>), grid, dim3(kDxThreads), lds, s, a);
-  else hipLaunchKernelGGL((dxrows_kernel<f16_t, CT>), grid, dim3(kDxThreads), lds, s, a);
+  if (x_dtype == CAIFX_F32) hipLaunchKernelGGL((dxrows_kernel<float, CT, kInt4>), grid, dim3(kDxThreads), lds, s, a);
+  else if (x_dtype == CAIFX_BF16) hipLaunchKernelGGL((dxrows_kernel<bf16_t, CT, kInt4>), grid, dim3(kDxThreads), lds, s, a);
+  else hipLaunchKernelGGL((dxrows_kernel<f16_t, CT, kInt4>), grid, dim3(kDxThreads), lds, s, a);
   return launch_status();
+}
+
+template <typename CT>
+int launch_ct(const DxArgs &a, bool int4, int x_dtype, dim3 grid, size_t lds, hipStream_t s)
+{
+  return int4 ? launch_xt<CT, true>(a, x_dtype, grid, lds, s) : launch_xt<CT, false>(a, x_dtype, grid, lds, s);
 }
 
 struct DxPlan {
   bool ok;
   int period;
+  int group_shift;
   int64_t rows_per_wg;
   int64_t ranges;          // workgroups along the rows
 };
 
 DxPlan plan(const GemmArgs &g)
 {
-  DxPlan p{false, 0, 0, 0};
-  if (g.offsets || g.M < 1 || g.M > 16 || g.w.kind != CAIFX_W_INT8) return p;
+  DxPlan p{false, 0, 0, 0, 0};
+  if (g.offsets || g.M < 1 || g.M > 16 || (g.w.kind != CAIFX_W_INT8 && g.w.kind != CAIFX_W_INT4_GROUP)) return p;
   if (g.K % kDxSlab != 0 || g.N < 1 || g.N > (int64_t{1} << 30) || g.K > (int64_t{1} << 30)) return p;
-  if (g.w.scales && g.w.scale_period > 1) {
+  if (g.w.kind == CAIFX_W_INT4_GROUP) {
+    // groups of 128 or more (a power of two): a slab of 128 columns has one scale per row.  (The size query
+    // comes without a group size and is answered for such groups.)
+    const int gs = g.w.group_size;
+    if (gs != 0 && (gs < kDxSlab || (gs & (gs - 1)) != 0)) return p;
+    p.group_shift = gs != 0 ? __builtin_ctz(static_cast<unsigned>(gs)) : 7;
+  } else if (g.w.scales && g.w.scale_period > 1) {
     if (g.K % g.w.scale_period != 0) return p;       // the scale would depend on the weight row
     p.period = static_cast<int>(g.w.scale_period);
   } else if (g.w.scales) {
@@ -213,13 +246,15 @@ int dxrows_backward(const GemmArgs &g, hipStream_t s)
 {
   const DxPlan p = plan(g);
   if (!p.ok) return CAIFX_ERR_UNSUPPORTED;
-  if (!aligned_to(g.w.q, 8) || (g.w.scales && !aligned_to(g.w.scales, 4))) return CAIFX_ERR_UNSUPPORTED;
+  const bool int4 = g.w.kind == CAIFX_W_INT4_GROUP;
+  if (int4 && (!g.w.scales || g.w.group_size == 0)) return CAIFX_ERR_UNSUPPORTED;
+  if (!aligned_to(g.w.q, 8) || (g.w.scales && !aligned_to(g.w.scales, int4 ? 2 : 4))) return CAIFX_ERR_UNSUPPORTED;
   const bool split = p.ranges > 1;
   if (split && (!g.workspace || !aligned_to(g.workspace, 4) || g.workspace_bytes < dxrows_workspace_bytes(g)))
     return CAIFX_ERR_UNSUPPORTED;
   DxArgs a{};
   a.wq = static_cast<const int8_t *>(g.w.q);
-  a.scales = static_cast<const float *>(g.w.scales);
+  a.scales = g.w.scales;
   a.dy = g.x;
   a.dx = g.y;
   a.M = static_cast<int>(g.M);
@@ -227,13 +262,14 @@ int dxrows_backward(const GemmArgs &g, hipStream_t s)
   a.N = g.N;
   a.K = g.K;
   a.period = p.period;
+  a.group_shift = p.group_shift;
   a.rows_per_wg = p.rows_per_wg;
   a.partial = split ? static_cast<float *>(g.workspace) : nullptr;
   const dim3 grid(static_cast<unsigned>(g.K / kDxSlab), static_cast<unsigned>(p.ranges));
   const size_t lds = static_cast<size_t>(kDxWaves) * 8 * 4 * 64 * sizeof(float);
-  const int st = g.compute_dtype == CAIFX_F32 ? launch_ct<float>(a, g.x_dtype, grid, lds, s)
-                 : g.compute_dtype == CAIFX_BF16 ? launch_ct<bf16_t>(a, g.x_dtype, grid, lds, s)
-                                                 : launch_ct<f16_t>(a, g.x_dtype, grid, lds, s);
+  const int st = g.compute_dtype == CAIFX_F32 ? launch_ct<float>(a, int4, g.x_dtype, grid, lds, s)
+                 : g.compute_dtype == CAIFX_BF16 ? launch_ct<bf16_t>(a, int4, g.x_dtype, grid, lds, s)
+                                                 : launch_ct<f16_t>(a, int4, g.x_dtype, grid, lds, s);
   if (st != CAIFX_OK || !split) return st;
   return splitk_reduce(a.partial, static_cast<int>(p.ranges), g.M * g.K, g.y, g.y_dtype, nullptr, s);
 }

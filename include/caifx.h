@@ -146,9 +146,10 @@ CAIFX_API int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K,
  * (src/caif_device_frozen_linear.cpp:549-645): replaces ConvertToComputeDtype()
  * + grad.To(ComputeT) + cublasGemmEx / CAIF_Ops::MatMul.
  *   dX[M,K] = cast<compute>(dY)[M,N] * cast<compute>(dequant(W))[N,K], fp32 accumulate.
- * With up to 16 rows, int8 codes and a scale that does not depend on the weight row (K a multiple of
- * scale_period, one scale, or none) the weight is streamed once through the fp32 matrix core and its scale is
- * applied to the finished column: like the forward's memory-bound kernels this skips the rounding of
+ * With up to 16 rows and int8 codes whose scale does not depend on the weight row (K a multiple of
+ * scale_period, one scale, or none) or int4 codes in groups of 128 or more, the weight is streamed once through
+ * the fp32 matrix core and its scale is applied outside the products: like the forward's memory-bound kernels
+ * this skips the rounding of
  * code * scale to a 16-bit compute type (about 2e-3 of max|dX| for bf16; for the fp32 compute type the
  * difference is fp32 rounding, 1e-7). */
 CAIFX_API int caifx_qlinear_backward_input(int64_t M, int64_t N, int64_t K,
@@ -186,7 +187,7 @@ CAIFX_API int caifx_qlinear_backward_input_add(int64_t M, int64_t N, int64_t K,
  * not depend on scheduling).  The fp32 compute type does the same for up to 128 rows.  The forward with up to
  * 32 rows cuts a reduction longer than one workgroup covers into slices whose sums meet there (K > 4096 with up
  * to 16 rows, K > 2048 with 17..32 rows or with int8 codes and N small enough that the activations' preparation
- * outweighs a workgroup's share of the weight), and the input gradient with up to 16 rows of int8 codes splits
+ * outweighs a workgroup's share of the weight), and the input gradient with up to 16 rows splits
  * the weight's rows among workgroups the same way.  With a smaller or null
  * workspace the calls run without that sharing, only slower, and the sums are formed in a different order, so
  * the last bits of a result may differ between a call with and a call without the workspace. */

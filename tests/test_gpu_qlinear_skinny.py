@@ -311,11 +311,12 @@ def _check_dx(orc, rng, M, N, K, kind, cd, xd, yd=0, workspace=None):
     return err
 
 
-@pytest.mark.parametrize("kind", ["int8pc", "int8pt", "int8raw"])
+@pytest.mark.parametrize("kind", ["int8pc", "int8pt", "int8raw", "int4"])
 @pytest.mark.parametrize("M", [1, 5, 16])
 def test_input_gradient_few_rows_fp32(orc, kind, M):
-    # dX = dY W for up to 16 rows of int8 codes streams the weight once through the fp32 matrix core when the scale
-    # of W[n][k] does not depend on n (square per-channel weight: K mod N = 0; one scale; none).  Shapes: BASELINE
+    # dX = dY W for up to 16 rows streams the weight once through the fp32 matrix core: int8 codes when the scale
+    # of W[n][k] does not depend on n (square per-channel weight: K mod N = 0; one scale; none), int4 codes in
+    # groups of 128 or more (the scale of a row and group rides on the gradient).  Shapes: BASELINE
     # config 1 (4096 x 4096), a row count that is no multiple of a wave's 16 rows (N = 1000), a single column slab
     # (K = 128), fewer rows than one workgroup pass (N = 40).
     rng = np.random.default_rng(300 + M)
@@ -330,19 +331,21 @@ def test_input_gradient_few_rows_dtype_mixes(orc, cd, xd, yd):
     # 16-bit compute types: dY is rounded to the compute type first (the layer's cast of its input); the weight is
     # not (post-scaled class, like the decode forward)
     rng = np.random.default_rng(cd * 9 + xd * 3 + yd)
-    for kind, N, K in (("int8pc", 512, 1024), ("int8pt", 777, 384)):
+    for kind, N, K in (("int8pc", 512, 1024), ("int8pt", 777, 384), ("int4", 640, 1280)):
         err = _check_dx(orc, rng, 7, N, K, kind, cd, xd, yd)
         if cd != 0 and yd == 0:
             assert err <= TIGHT_POST
 
 
 def test_input_gradient_few_rows_other_paths(orc):
-    # per-channel scales whose index depends on the weight row (K mod N != 0), int4 codes, more than 16 rows and a
-    # call without a workspace go to the tiled kernels; all must agree with the oracle
+    # per-channel scales whose index depends on the weight row (K mod N != 0), int4 groups below 128, more than 16
+    # rows and a call without a workspace go to the tiled kernels; all must agree with the oracle
     import torch
     rng = np.random.default_rng(31)
     _check_dx(orc, rng, 8, 1536, 1024, "int8pc", 0, 0)
-    _check_dx(orc, rng, 8, 512, 1024, "int4", 2, 2)
+    ow, dw = make_weight(orc, rng, 512, 1024, "int4", 64)
+    dy = dev_as(rng.normal(0, 1e-3, (8, 512)), 2)
+    assert max_rel_err(host(T.qlinear_backward_input(dy, dw, 2)), orc.frozen_linear_backward(host(dy), ow, 2)) <= TIGHT_16
     _check_dx(orc, rng, 17, 512, 512, "int8pc", 0, 0)
     none = torch.empty(0, dtype=torch.uint8, device="cuda")
     _check_dx(orc, rng, 16, 2048, 2048, "int8pc", 0, 0, workspace=none)
