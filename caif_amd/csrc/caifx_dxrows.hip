@@ -8,8 +8,9 @@
 // exact in fp32 and the weight's scale is applied to the finished column, so nothing is rounded to a 16-bit type
 // on the way (the reference rounds code*scale to the compute dtype first; results differ by that rounding, a
 // few 1e-3 of the largest output for bf16, 1e-7 for the fp32 compute type).
-// That needs the scale of W[n][k] not to depend on n: scale index (n*K + k) mod period with K a multiple of the
-// period (which covers the per-output-channel scales of a square weight), one scale, or none.
+// That needs the scale of W[n][k] not to depend on n among the rows a workgroup visits: scale index
+// (n*K + k) mod period with K a multiple of the period (the per-output-channel scales of a square weight), one
+// scale, none, or any period with the rows split into residue classes (see DxArgs::V).
 // Packed int4 codes in groups of 128 or more take the same route with the scale on the other operand: a slab of
 // 128 columns lies inside one group, so the scale of (row, group) multiplies the row's gradient before it enters
 // the A operand.
@@ -43,7 +44,12 @@ struct DxArgs {
   int64_t N, K;
   int period;              // int8: 0: no scale, 1: scales[0], else scales[k % period]
   int group_shift;         // int4: log2 of the group size (>= 7: a slab lies inside one group)
-  int64_t rows_per_wg;     // rows of W per blockIdx.y
+  // int8 scale vectors whose index depends on the weight row: rows n with equal n mod V see the same scales along
+  // k (V = period / gcd(K mod period, period)), so a workgroup only visits rows n = cls + V*i of one residue class
+  // and its columns still have one scale each, scales[(cls*K + k) mod period].  V = 1 otherwise.
+  int V;
+  int ranges;              // row ranges per class: blockIdx.y = cls * ranges + range
+  int64_t rows_per_wg;     // rows of a class per workgroup
   float *partial;          // [gridDim.y][M][K] when the rows are split among workgroups, else null
 };
 
@@ -59,8 +65,10 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
   const int j = lane & 15;
   const int q = lane >> 4;
   const int64_t k0 = static_cast<int64_t>(blockIdx.x) * kDxSlab;
-  const int64_t n_lo = static_cast<int64_t>(blockIdx.y) * a.rows_per_wg;
-  const int64_t n_hi = n_lo + a.rows_per_wg < a.N ? n_lo + a.rows_per_wg : a.N;
+  const int cls = blockIdx.y / a.ranges;
+  const int64_t rows_class = (a.N - cls + a.V - 1) / a.V;              // rows n = cls + V*i, i < rows_class
+  const int64_t n_lo = static_cast<int64_t>(blockIdx.y - cls * a.ranges) * a.rows_per_wg;      // (i, not n, from here on)
+  const int64_t n_hi = n_lo + a.rows_per_wg < rows_class ? n_lo + a.rows_per_wg : rows_class;
   const XT *dy = static_cast<const XT *>(a.dy) + static_cast<int64_t>(j < a.M ? j : a.M - 1) * a.N;
   const int8_t *wcol = a.wq + (kInt4 ? (k0 >> 1) + 4 * j : k0 + 8 * j);
   const int64_t row_bytes = kInt4 ? a.K >> 1 : a.K;
@@ -83,7 +91,7 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
 #pragma unroll
     for (int it = 0; it < kDxIter; ++it) {
       const int64_t n = base + 4 * it + q;
-      const int64_t nn = n < n_hi ? n : n_hi - 1;          // rows past the range: a valid address, a zero gradient
+      const int64_t nn = cls + a.V * (n < n_hi ? n : n_hi - 1);          // rows past the range: a valid address, a zero gradient
       if constexpr (kInt4) {
         w[st][it][0] = *reinterpret_cast<const uint32_t *>(wcol + nn * row_bytes);
         ws[st][it] = s16[(nn * a.K + k0) >> a.group_shift];
@@ -160,7 +168,7 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
     if constexpr (!kInt4) {
       const float *s32 = static_cast<const float *>(a.scales);
       if (a.period == 1) s = s32[0];
-      else if (a.period > 1) s = s32[k % a.period];
+      else if (a.period > 1) s = s32[(static_cast<int64_t>(cls) * a.K + k) % a.period];
     }
     const float v = tiles[o] * s;
     const int64_t at = static_cast<int64_t>(m) * a.K + k;
@@ -198,13 +206,14 @@ struct DxPlan {
   bool ok;
   int period;
   int group_shift;
+  int V;                   // residue classes of the rows (int8 scale vectors), else 1
   int64_t rows_per_wg;
-  int64_t ranges;          // workgroups along the rows
+  int64_t ranges;          // workgroups along the rows of a class
 };
 
 DxPlan plan(const GemmArgs &g)
 {
-  DxPlan p{false, 0, 0, 0, 0};
+  DxPlan p{false, 0, 0, 1, 0, 0};
   if (g.offsets || g.M < 1 || g.M > 16 || (g.w.kind != CAIFX_W_INT8 && g.w.kind != CAIFX_W_INT4_GROUP)) return p;
   if (g.K % kDxSlab != 0 || g.N < 1 || g.N > (int64_t{1} << 30) || g.K > (int64_t{1} << 30)) return p;
   if (g.w.kind == CAIFX_W_INT4_GROUP) {
@@ -214,32 +223,58 @@ DxPlan plan(const GemmArgs &g)
     if (gs != 0 && (gs < kDxSlab || (gs & (gs - 1)) != 0)) return p;
     p.group_shift = gs != 0 ? __builtin_ctz(static_cast<unsigned>(gs)) : 7;
   } else if (g.w.scales && g.w.scale_period > 1) {
-    if (g.K % g.w.scale_period != 0) return p;       // the scale would depend on the weight row
-    p.period = static_cast<int>(g.w.scale_period);
+    const int64_t P = g.w.scale_period;
+    if (P > (int64_t{1} << 30)) return p;
+    int64_t a = g.K % P == 0 ? P : g.K % P, b = P;       // V = P / gcd(K mod P, P)
+    while (b) {
+      const int64_t t = a % b;
+      a = b;
+      b = t;
+    }
+    const int64_t V = P / a;
+    if (V > 64 || V * kDxPassRows > g.N) return p;       // too many classes, or too few rows in each
+    p.V = static_cast<int>(V);
+    p.period = static_cast<int>(P);
   } else if (g.w.scales) {
     p.period = 1;
   }
   const int64_t slabs = g.K / kDxSlab;
   static const int cus = compute_units();
-  int64_t ranges = (cus + slabs - 1) / slabs;
-  const int64_t most = (g.N + kDxPassRows - 1) / kDxPassRows;      // every workgroup gets at least one full pass
+  const int64_t rows_class = (g.N + p.V - 1) / p.V;                 // of the largest class
+  int64_t ranges = (cus + slabs * p.V - 1) / (slabs * p.V);
+  const int64_t most = (rows_class + kDxPassRows - 1) / kDxPassRows;      // every workgroup gets at least one full pass
   if (ranges > most) ranges = most;
-  if (ranges > 65535) ranges = 65535;
-  int64_t rows = (g.N + ranges - 1) / ranges;
+  if (ranges < 1) ranges = 1;
+  int64_t rows = (rows_class + ranges - 1) / ranges;
   rows = (rows + kDxWaveRows - 1) / kDxWaveRows * kDxWaveRows;
   p.rows_per_wg = rows;
-  p.ranges = (g.N + rows - 1) / rows;
-  p.ok = slabs <= 0x7fffffff;
+  p.ranges = (rows_class + rows - 1) / rows;
+  p.ok = slabs <= 0x7fffffff && p.ranges * p.V <= 65535;
   return p;
 }
 
 }  // namespace
 
-size_t dxrows_workspace_bytes(const GemmArgs &g)
+static size_t plan_bytes(const GemmArgs &g)
 {
   const DxPlan p = plan(g);
-  if (!p.ok || p.ranges < 2) return 0;
-  return static_cast<size_t>(p.ranges) * static_cast<size_t>(g.M) * static_cast<size_t>(g.K) * sizeof(float);
+  if (!p.ok || p.ranges * p.V < 2) return 0;
+  return static_cast<size_t>(p.ranges * p.V) * static_cast<size_t>(g.M) * static_cast<size_t>(g.K) * sizeof(float);
+}
+
+size_t dxrows_workspace_bytes(const GemmArgs &g)
+{
+  size_t bytes = plan_bytes(g);
+  if (g.w.kind == CAIFX_W_INT8 && !g.w.scales) {
+    // a size query knows no scales: also cover a vector of one scale per output feature (period N), the usual
+    // int8 layout, whose residue classes each bring their own partial sums
+    GemmArgs c = g;
+    c.w.scales = &c;              // any non-null address; only its presence is looked at
+    c.w.scale_period = g.N;
+    const size_t per_feature = plan_bytes(c);
+    if (per_feature > bytes) bytes = per_feature;
+  }
+  return bytes;
 }
 
 int dxrows_backward(const GemmArgs &g, hipStream_t s)
@@ -249,7 +284,7 @@ int dxrows_backward(const GemmArgs &g, hipStream_t s)
   const bool int4 = g.w.kind == CAIFX_W_INT4_GROUP;
   if (int4 && (!g.w.scales || g.w.group_size == 0)) return CAIFX_ERR_UNSUPPORTED;
   if (!aligned_to(g.w.q, 8) || (g.w.scales && !aligned_to(g.w.scales, int4 ? 2 : 4))) return CAIFX_ERR_UNSUPPORTED;
-  const bool split = p.ranges > 1;
+  const bool split = p.ranges * p.V > 1;
   if (split && (!g.workspace || !aligned_to(g.workspace, 4) || g.workspace_bytes < dxrows_workspace_bytes(g)))
     return CAIFX_ERR_UNSUPPORTED;
   DxArgs a{};
@@ -264,14 +299,16 @@ int dxrows_backward(const GemmArgs &g, hipStream_t s)
   a.period = p.period;
   a.group_shift = p.group_shift;
   a.rows_per_wg = p.rows_per_wg;
+  a.V = p.V;
+  a.ranges = static_cast<int>(p.ranges);
   a.partial = split ? static_cast<float *>(g.workspace) : nullptr;
-  const dim3 grid(static_cast<unsigned>(g.K / kDxSlab), static_cast<unsigned>(p.ranges));
+  const dim3 grid(static_cast<unsigned>(g.K / kDxSlab), static_cast<unsigned>(p.ranges * p.V));
   const size_t lds = static_cast<size_t>(kDxWaves) * 8 * 4 * 64 * sizeof(float);
   const int st = g.compute_dtype == CAIFX_F32 ? launch_ct<float>(a, int4, g.x_dtype, grid, lds, s)
                  : g.compute_dtype == CAIFX_BF16 ? launch_ct<bf16_t>(a, int4, g.x_dtype, grid, lds, s)
                                                  : launch_ct<f16_t>(a, int4, g.x_dtype, grid, lds, s);
   if (st != CAIFX_OK || !split) return st;
-  return splitk_reduce(a.partial, static_cast<int>(p.ranges), g.M * g.K, g.y, g.y_dtype, nullptr, s);
+  return splitk_reduce(a.partial, static_cast<int>(p.ranges * p.V), g.M * g.K, g.y, g.y_dtype, nullptr, s);
 }
 
 }  // namespace caifx

@@ -55,9 +55,8 @@ int mblock_grouped_forward(const GemmArgs &a, hipStream_t s);
 // Workspace of mblock_forward when the reduction is longer than one workgroup covers (K > 4096), else 0.
 size_t mblock_workspace_bytes(const GemmArgs &a);
 
-// Input gradient for M <= 16 rows of dY with int8 codes whose scale index does not depend on the weight row
-// (K a multiple of the scale period, one scale, or none) or int4 codes in groups of 128 or more, on the fp32
-// matrix core.  Needs the workspace
+// Input gradient for M <= 16 rows of dY with int8 codes (scale vectors through residue classes of the rows, one
+// scale, or none) or int4 codes in groups of 128 or more, on the fp32 matrix core.  Needs the workspace
 // dxrows_workspace_bytes reports when that is not 0; CAIFX_ERR_UNSUPPORTED otherwise.
 int dxrows_backward(const GemmArgs &a, hipStream_t s);
 size_t dxrows_workspace_bytes(const GemmArgs &a);

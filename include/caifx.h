@@ -146,8 +146,9 @@ CAIFX_API int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K,
  * (src/caif_device_frozen_linear.cpp:549-645): replaces ConvertToComputeDtype()
  * + grad.To(ComputeT) + cublasGemmEx / CAIF_Ops::MatMul.
  *   dX[M,K] = cast<compute>(dY)[M,N] * cast<compute>(dequant(W))[N,K], fp32 accumulate.
- * With up to 16 rows and int8 codes whose scale does not depend on the weight row (K a multiple of
- * scale_period, one scale, or none) or int4 codes in groups of 128 or more, the weight is streamed once through
+ * With up to 16 rows and int8 codes (any scale vector that leaves at most 64 residue classes of rows with
+ * equal scales along k, each of 256 rows or more; one scale; none) or int4 codes in groups of 128 or more, the
+ * weight is streamed once through
  * the fp32 matrix core and its scale is applied outside the products: like the forward's memory-bound kernels
  * this skips the rounding of
  * code * scale to a 16-bit compute type (about 2e-3 of max|dX| for bf16; for the fp32 compute type the

@@ -338,11 +338,11 @@ def test_input_gradient_few_rows_dtype_mixes(orc, cd, xd, yd):
 
 
 def test_input_gradient_few_rows_other_paths(orc):
-    # per-channel scales whose index depends on the weight row (K mod N != 0), int4 groups below 128, more than 16
-    # rows and a call without a workspace go to the tiled kernels; all must agree with the oracle
+    # per-channel scales whose index depends on the weight row in too many ways (205 residue classes), int4 groups
+    # below 128, more than 16 rows and a call without a workspace go to the tiled kernels; all must agree with the oracle
     import torch
     rng = np.random.default_rng(31)
-    _check_dx(orc, rng, 8, 1536, 1024, "int8pc", 0, 0)
+    _check_dx(orc, rng, 8, 2050, 640, "int8pc", 0, 0)
     ow, dw = make_weight(orc, rng, 512, 1024, "int4", 64)
     dy = dev_as(rng.normal(0, 1e-3, (8, 512)), 2)
     assert max_rel_err(host(T.qlinear_backward_input(dy, dw, 2)), orc.frozen_linear_backward(host(dy), ow, 2)) <= TIGHT_16
@@ -350,6 +350,15 @@ def test_input_gradient_few_rows_other_paths(orc):
     none = torch.empty(0, dtype=torch.uint8, device="cuda")
     _check_dx(orc, rng, 16, 2048, 2048, "int8pc", 0, 0, workspace=none)
     _check_dx(orc, rng, 3, 40, 128, "int8pt", 0, 0, workspace=none)     # one workgroup: no workspace needed
+
+
+@pytest.mark.parametrize("N,K,M", [(1536, 1024, 16), (14336, 4096, 4), (3584, 1024, 9)])
+def test_input_gradient_few_rows_residue_classes(orc, N, K, M):
+    # one scale per output feature with K mod N != 0: the scale of W[n][k] depends on n, but rows with equal
+    # n mod V (V = 3, 7, 7 here) share their scales along k; a workgroup stays inside one class
+    rng = np.random.default_rng(N + K + M)
+    assert _check_dx(orc, rng, M, N, K, "int8pc", 0, 0) <= 2e-6
+    assert _check_dx(orc, rng, M, N, K, "int8pc", 2, 2) <= TIGHT_POST
 
 
 def test_input_gradient_few_rows_is_the_adjoint_of_the_forward(orc):
