@@ -365,6 +365,18 @@ def compute_bound_rows(torch, T, dev, gen, capture, time_graph):
             rows[key].update({"dx_us": round(ms_b * 1e3, 2), "dx_TFLOPs": round(flops / (ms_b * 1e-3) / 1e12, 1),
                               "fwd_dx_frac_of_mfma_peak":
                                   round(2 * flops / ((ms_f + ms_b) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+        # yardstick, not part of the path: the vendor library's dense bf16 GEMM (torch.matmul) on the same shape with
+        # the weight already dequantised, i.e. what the platform's own kernel reaches without any unpacking
+        try:
+            wd = torch.empty(N, K, device=dev).normal_(0, 0.02, generator=gen).to(torch.bfloat16)
+            yd = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+            g = capture(lambda i: torch.matmul(x, wd.t(), out=yd), L)
+            ms_v = time_graph(g, L, reps=3)
+            del g, wd, yd
+            rows[key]["vendor_dense_bf16_fwd_TFLOPs"] = round(flops / (ms_v * 1e-3) / 1e12, 1)
+        except Exception as e:   # the yardstick must not take the row down
+            rows[key]["vendor_dense_bf16_fwd_TFLOPs"] = None
+            print(f"bench: vendor GEMM yardstick skipped: {type(e).__name__}: {e}", file=sys.stderr)
         if (M, N) == (4096, 11008):
             # configs[3]: what the LoRA adapter does with the frozen base around its own small GEMMs: the base
             # output cast to bf16 and added to the low-rank branch, forward and backward.  "chain" is the
