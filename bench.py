@@ -280,6 +280,22 @@ def decode_other_rows(torch, T, dev, gen, capture, time_graph):
             out["decode_down_proj"][f"{kind}_M{m}_N{N}_K{K}"] = {
                 "us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                 "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    # the input gradient with 16 rows through the same down-projection weights (dY [16, 4096] -> dX [16, 14336]):
+    # one pass over the weight on the fp32 matrix core, its row ranges meeting in the workspace
+    from caif_amd import capi
+    out["few_row_input_gradient"] = {}
+    dy = torch.empty(16, N, device=dev).normal_(0, 1e-3, generator=gen).to(torch.bfloat16)
+    dx = torch.empty(16, K, device=dev)
+    for kind, Ws, wk in (("int4", W4, T.W_INT4_GROUP), ("int8", W8, T.W_INT8)):
+        nb = capi.lib().caifx_qlinear_workspace_bytes(16, N, K, T.BF16, T.BF16, wk, 1)
+        wsb = torch.empty(max(nb, 1), dtype=torch.uint8, device=dev)
+        g = capture(lambda i, Ws=Ws: T.qlinear_backward_input(dy, Ws[i % len(Ws)], T.BF16, T.F32, out=dx, workspace=wsb), 40)
+        ms = time_graph(g, 40)
+        del g
+        nbytes = algorithmic_bytes(kind, 16, N=N, K=K)      # the same weight, 16 rows in, 16 rows out
+        out["few_row_input_gradient"][f"{kind}_M16_N{N}_K{K}"] = {
+            "us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     return out
 
 
