@@ -123,6 +123,35 @@ __device__ __forceinline__ void segment_rows(const int32_t *offsets, int e, int6
   hi = hi < lo ? lo : (hi > m ? m : hi);
 }
 
+// v_mfma_f32_32x32x16 in the 16-bit compute type CT: A is 32 rows x 16 (lane l supplies row l % 32, reduction
+// elements 8 * (l / 32) .. + 7), B likewise by column; of the 32 x 32 result lane l holds column l % 32 and, in
+// register r, row 8 * (r / 4) + 4 * (l / 32) + r % 4.
+template <typename CT> struct Mfma32;
+template <> struct Mfma32<bf16_t> {
+  typedef bf16x8_t vec_t;
+  static __device__ __forceinline__ floatx16_t run(vec_t a, vec_t b, floatx16_t c)
+  {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma32<f16_t> {
+  typedef f16x8_t vec_t;
+  static __device__ __forceinline__ floatx16_t run(vec_t a, vec_t b, floatx16_t c)
+  {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// two fp32 values rounded to CT (nearest even), the first in the low half
+template <typename CT> __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+{
+  typedef __attribute__((__vector_size__(2 * sizeof(CT)))) CT pair_t;
+  pair_t p;
+  p[0] = from_f32<CT>(lo);
+  p[1] = from_f32<CT>(hi);
+  return __builtin_bit_cast(uint32_t, p);
+}
+
 __device__ __forceinline__ float wave_max(float v)
 {
 #pragma unroll

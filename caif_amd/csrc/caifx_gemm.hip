@@ -25,6 +25,7 @@
 #include "caifx_internal.hpp"
 
 #include <atomic>
+#include <cstdlib>
 #include <type_traits>
 
 namespace caifx {
@@ -34,22 +35,6 @@ constexpr int BC = 128;      // columns of D per workgroup
 constexpr int BR = 64;       // reduction extent per step
 constexpr int kWStagers = 256;              // producer threads that stage the W piece (the first four producer waves)
 constexpr int kBTileBytes = BC * BR * 2;   // weight tile in LDS (16 KiB)
-
-template <typename CT> struct Mfma32;
-template <> struct Mfma32<bf16_t> {
-  typedef bf16x8_t vec_t;
-  static __device__ __forceinline__ floatx16_t run(vec_t a, vec_t b, floatx16_t c)
-  {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-};
-template <> struct Mfma32<f16_t> {
-  typedef f16x8_t vec_t;
-  static __device__ __forceinline__ floatx16_t run(vec_t a, vec_t b, floatx16_t c)
-  {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  }
-};
 
 enum { SM_SCALAR = 0, SM_VEC4 = 1, SM_ANY = 2 };   // how int8 scales are fetched
 // What the store does besides rounding the accumulator v to the result type T:
@@ -90,15 +75,6 @@ struct TileArgs {
 // with bits of the row so that (a) 8 consecutive rows at one chunk index and (b) rows 8 apart at one
 // chunk index (the transposed weight writes of the backward case) land in different banks.
 __device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + ((chunk ^ ((row ^ (row >> 3)) & 7)) << 4); }
-
-template <typename CT> __device__ __forceinline__ uint32_t pack2(float lo, float hi)
-{
-  typedef __attribute__((__vector_size__(2 * sizeof(CT)))) CT pair_t;
-  pair_t p;
-  p[0] = from_f32<CT>(lo);
-  p[1] = from_f32<CT>(hi);
-  return __builtin_bit_cast(uint32_t, p);
-}
 
 __device__ __forceinline__ float int8_scale_at(const float *scales, int mode, int64_t period, int64_t flat)
 {
@@ -926,7 +902,15 @@ int splitk_reduce(const float *partial, int parts, int64_t n, void *y, int y_dty
   return launch_status();
 }
 
-int mfma_forward(const GemmArgs &a, hipStream_t s) { return run(a, false, s); }
+int mfma_forward(const GemmArgs &a, hipStream_t s)
+{
+#ifdef CAIFX_DEV
+  const char *sw = getenv("CAIFX_REGW");
+  if (sw && sw[0] == '0') return run(a, false, s);
+#endif
+  const int st = mfma_regw_forward(a, s);
+  return st == CAIFX_ERR_UNSUPPORTED ? run(a, false, s) : st;
+}
 int mfma_backward(const GemmArgs &a, hipStream_t s) { return run(a, true, s); }
 size_t mfma_workspace_bytes(const GemmArgs &a, bool backward)
 {

@@ -65,6 +65,10 @@ size_t dxrows_workspace_bytes(const GemmArgs &a);
 int mfma_forward(const GemmArgs &a, hipStream_t s);
 int mfma_backward(const GemmArgs &a, hipStream_t s);
 size_t mfma_workspace_bytes(const GemmArgs &a, bool backward);
+// Forward for packed int4 weights and 16-bit activations of the compute type with enough 128 x 256 tiles to fill
+// the chip: the weight goes from global memory straight into matrix-core operand registers.
+// CAIFX_ERR_UNSUPPORTED for everything else (mfma_forward tries it first).
+int mfma_regw_forward(const GemmArgs &a, hipStream_t s);
 
 // fp32 compute type on the matrix cores (v_mfma_f32_32x32x2_f32), forward and input gradient, any M, plain
 // and grouped.  CAIFX_ERR_UNSUPPORTED for an addend, reductions that are not a multiple of 32,
