@@ -259,6 +259,35 @@ def decode_other_rows(torch, T, dev, gen, capture, time_graph):
         out["decode_tall_M1"][kind] = {"N": N_TALL, "copies_rotated": len(fws), "us": round(ms * 1e3, 2),
                                        "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                        "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    # yardstick, not part of the path: what kernels that are not this library's read per second from the same
+    # rotated buffers (each launch a different 470 MB copy, so nothing comes from cache): a sum over the bytes
+    # (one pass of reads, nothing written) and a device-to-device copy (half reads, half writes)
+    try:
+        bufs = [fw.wq for fw in tall[1][1]]
+        nb = bufs[0].numel()
+        views = [b.view(torch.int32) for b in bufs]
+        sink = torch.empty(nb, dtype=torch.int8, device=dev)
+        acc = torch.zeros((), dtype=torch.int64, device=dev)
+
+        def timed(fn, n=6):
+            fn(0)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(n):
+                fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / n
+
+        ms_sum = timed(lambda i: acc.copy_(views[i % len(views)].sum(dtype=torch.int64)))
+        ms_cpy = timed(lambda i: sink.copy_(bufs[i % len(bufs)]))
+        out["hbm_stream_yardstick_GBps"] = {"bytes": nb, "torch_sum_read_only": round(nb / (ms_sum * 1e-3) / 1e9, 1),
+                                            "device_copy_read_plus_write": round(2 * nb / (ms_cpy * 1e-3) / 1e9, 1)}
+        del bufs, views, sink, acc
+    except Exception as e:   # a yardstick must not take the rows down
+        out["hbm_stream_yardstick_GBps"] = None
+        print(f"bench: HBM stream yardstick skipped: {type(e).__name__}: {e}", file=sys.stderr)
     del tall, fws
     del p4, s4, q8, s8, y
     N, K = 4096, 14336
@@ -393,6 +422,27 @@ def compute_bound_rows(torch, T, dev, gen, capture, time_graph):
         except Exception as e:   # the yardstick must not take the row down
             rows[key]["vendor_dense_bf16_fwd_TFLOPs"] = None
             print(f"bench: vendor GEMM yardstick skipped: {type(e).__name__}: {e}", file=sys.stderr)
+        # second yardstick: the matrix pipes alone (no loads, stores or unpacking) on this row's own values.  Their
+        # clock follows the power the operand bit patterns draw, so this, not the published peak, is what a kernel
+        # that did everything else for free would reach on N(0,1) activations and N(0,0.02) weights
+        try:
+            wvals = torch.empty(16384, device=dev).normal_(0, 0.02, generator=gen)
+            iters = 600
+            fl, keep = T.probe_mfma_bf16(x, wvals, iters)         # untimed: clocks settle
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(3):
+                fl, keep = T.probe_mfma_bf16(x, wvals, iters)
+            e1.record()
+            torch.cuda.synchronize()
+            pipes = 3 * fl / (e0.elapsed_time(e1) * 1e-3) / 1e12
+            rows[key]["mfma_pipes_alone_on_these_values_TFLOPs"] = round(pipes, 1)
+            rows[key]["fwd_frac_of_pipes_alone"] = round(rows[key]["fwd_TFLOPs"] / pipes, 4)
+            del keep, wvals
+        except Exception as e:
+            rows[key]["mfma_pipes_alone_on_these_values_TFLOPs"] = None
+            print(f"bench: matrix-pipe yardstick skipped: {type(e).__name__}: {e}", file=sys.stderr)
         if (M, N) == (4096, 11008):
             # configs[3]: what the LoRA adapter does with the frozen base around its own small GEMMs: the base
             # output cast to bf16 and added to the low-rank branch, forward and backward.  "chain" is the
@@ -564,6 +614,51 @@ def moe_rows(torch, T, dev, gen):
 
     ms_f, ms_b = timed(fwd), timed(bwd)
     ms_f_fused, ms_b_fused = timed(fwd_gating_in_store), timed(bwd_gating_in_store)
+
+    # Per-expert-segment GEMM efficiency (outside the timed runs): the grouped kernel stamps every 128 x 128 tile
+    # with its expert, row count, start and end (100 MHz wall clock).  An expert's efficiency is the flops of its
+    # segment over what the matrix pipes offer during its tiles' lifetimes, 2 cnt K N / (sum of tile durations x
+    # peak / (256 compute units x 2 workgroups that share one)); partial last tiles and everything a tile waits
+    # for count against it.
+    def segment_efficiency(launch, n_cols, k_red):
+        from caif_amd import capi
+        tiles = ((rows + 127) // 128 + E) * ((n_cols + 127) // 128)
+        stamps = torch.zeros(tiles * 4, dtype=torch.int64, device=dev)
+        capi.call("caifx_qlinear_grouped_tile_stamps", stamps.data_ptr(), tiles)
+        try:
+            launch()
+            torch.cuda.synchronize()
+        finally:
+            capi.call("caifx_qlinear_grouped_tile_stamps", None, 0)
+        st = stamps.view(-1, 4).cpu()
+        st = st[st[:, 3] > 0]
+        cnt = counts.cpu()
+        share = MFMA_BF16_PEAK_TFLOPS * 1e12 / (256 * 2)
+        effs = []
+        for e in range(E):
+            mine = st[st[:, 0] == e]
+            if len(mine) == 0 or int(cnt[e]) == 0:
+                continue
+            busy_s = float((mine[:, 3] - mine[:, 2]).sum()) / 1e8
+            effs.append(2.0 * int(cnt[e]) * n_cols * k_red / (busy_s * share))
+        effs.sort()
+        span_s = float(st[:, 3].max() - st[:, 2].min()) / 1e8
+        return {"experts": len(effs), "tiles": int(len(st)), "min": round(effs[0], 4), "median": round(effs[len(effs) // 2], 4),
+                "max": round(effs[-1], 4), "first_start_to_last_end_us": round(span_s * 1e6, 1)}
+
+    try:
+        seg = {"definition": "2*rows_e*K*N / (sum of the expert's tile durations * 2.5 PFLOP/s / 512 resident workgroups)",
+               "gate_forward_2048_to_1408": segment_efficiency(
+                   lambda: T.qlinear_grouped_forward(x, offsets, gate, T.BF16, T.BF16, out=gate_o, workspace=ws), H, D),
+               "down_forward_1408_to_2048": segment_efficiency(
+                   lambda: T.qlinear_grouped_forward(hidden, offsets, down, T.BF16, T.BF16, out=out, workspace=ws), D, H),
+               "down_input_gradient": segment_efficiency(
+                   lambda: T.qlinear_grouped_backward_input(gout, offsets, down, T.BF16, T.BF16, out=gh, workspace=ws), H, D),
+               "gate_input_gradient": segment_efficiency(
+                   lambda: T.qlinear_grouped_backward_input(grad_gate, offsets, gate, T.BF16, T.BF16, out=gi_gate,
+                                                            workspace=ws), D, H)}
+    except Exception as e:   # a diagnostic must not take the row down
+        seg = {"error": repr(e)}
     # token routing around the experts (dispatch map, gather, weighted combine, and their backward passes),
     # on the same routing; HBM-bound row moves: algorithmic bytes = rows read + rows written
     idx2 = ids.reshape(tokens, top_k).to(torch.int32).contiguous()
@@ -618,6 +713,7 @@ def moe_rows(torch, T, dev, gen):
             "tokens_per_s_fwd_bwd_with_routing": round(tokens / ((ms_f + ms_b + routing_ms) * 1e-3), 1),
             "grouped_gemm_TFLOPs_fwd": round(gemm_flops / (ms_f * 1e-3) / 1e12, 1),
             "grouped_gemm_TFLOPs_bwd": round(gemm_flops / (ms_b * 1e-3) / 1e12, 1),
+            "per_expert_segment_gemm_efficiency": seg,
             "grouped_frac_of_mfma_peak": round(2 * gemm_flops / ((ms_f + ms_b) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
             # the other bound of a pass: every expert weight (int8 codes + fp32 per-channel scales) streamed once
             "weight_bytes_per_pass": int(3 * E * D * H + E * (2 * H + D) * 4),

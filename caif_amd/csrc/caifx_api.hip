@@ -348,6 +348,13 @@ static int grouped(bool backward, int num_experts, const int32_t *offsets, int64
   return backward ? generic_backward(a, s) : generic_forward(a, s);
 }
 
+int caifx_qlinear_grouped_tile_stamps(void *stamps, int64_t tiles)
+{
+  if (tiles < 0 || (stamps && !aligned_to(stamps, 8))) return CAIFX_ERR_INVALID_ARGUMENT;
+  mfma_grouped_tile_stamps(stamps, tiles);
+  return CAIFX_OK;
+}
+
 int caifx_qlinear_grouped_forward(int num_experts, const int32_t *offsets, int64_t total_rows, int64_t N, int64_t K,
                                   const void *x, int x_dtype, int compute_dtype, const void *const *wq_ptrs,
                                   int w_kind, const void *const *scales_ptrs, int64_t scale_period, int group_size,

@@ -25,7 +25,6 @@
 #include "caifx_internal.hpp"
 
 #include <atomic>
-#include <cstdlib>
 #include <type_traits>
 
 namespace caifx {
@@ -69,6 +68,9 @@ struct TileArgs {
   // reduction and writes its fp32 partial tile to d + split * M * C (d is then the caller's workspace)
   int ksplit;
   int split_steps;
+  // grouped form, measurement only: per tile {expert, rows, start, end} in 100 MHz ticks (null: nothing is recorded)
+  unsigned long long *stamps;
+  long long stamps_capacity;
 };
 
 // byte offset of 16-byte chunk `chunk` (0..7) of LDS tile row `row`.  The chunk position is XORed
@@ -115,6 +117,7 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
   // ---- which tile -----------------------------------------------------------------------
   int64_t row_lo, row_hi;        // rows of A / D this workgroup may touch: [row_lo, row_hi)
   int split = 0;                 // which part of the reduction (plain form with ksplit > 1)
+  int64_t stamp_pos = -1;        // grouped form with a stamp buffer: thread 0 writes the tile's end time there
   int64_t col_tile = blockIdx.x;
   const uint8_t *wq = static_cast<const uint8_t *>(g.wq);
   const void *scales = g.scales;
@@ -178,6 +181,13 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
     row_hi = hi;
     wq = static_cast<const uint8_t *>(g.wq_ptrs[e]);
     scales = g.scales_ptrs ? g.scales_ptrs[e] : nullptr;
+    if (g.stamps && threadIdx.x == 0 && pos < g.stamps_capacity) {
+      const int64_t rows = row_hi - row_lo < BM ? row_hi - row_lo : BM;
+      g.stamps[4 * pos] = static_cast<unsigned long long>(e);
+      g.stamps[4 * pos + 1] = static_cast<unsigned long long>(rows);
+      g.stamps[4 * pos + 2] = wall_clock64();
+      stamp_pos = pos;
+    }
   } else {
     // Workgroups are handed to the 8 XCDs in turn (linear id mod 8), and each XCD has its own L2.
     // The tiles are therefore numbered so that one XCD walks one contiguous eighth of the list, and
@@ -647,6 +657,9 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
     if (g.d_dtype == CAIFX_BF16) staged(bf16_t{});
     else if (g.d_dtype == CAIFX_F16) staged(f16_t{});
     else staged(float{});
+    if constexpr (kGrouped) {
+      if (stamp_pos >= 0) g.stamps[4 * stamp_pos + 3] = wall_clock64();      // thread 0 is in consumer wave 0
+    }
     return;
   }
 #pragma unroll
@@ -674,6 +687,9 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kInt4 || 
         }
       }
     }
+  }
+  if constexpr (kGrouped) {
+    if (stamp_pos >= 0) g.stamps[4 * stamp_pos + 3] = wall_clock64();
   }
 }
 
@@ -804,6 +820,9 @@ SplitPlan plan_split(int64_t M, int64_t C, int64_t R, bool grouped)
   return p;
 }
 
+std::atomic<unsigned long long *> g_stamps{nullptr};
+std::atomic<long long> g_stamps_capacity{0};
+
 int run(const GemmArgs &a, bool backward, hipStream_t s)
 {
   if (a.compute_dtype == CAIFX_F32) return CAIFX_ERR_UNSUPPORTED;
@@ -863,6 +882,10 @@ int run(const GemmArgs &a, bool backward, hipStream_t s)
     }
   }
   t.ksplit = 1;
+  if (grouped) {
+    t.stamps = g_stamps.load(std::memory_order_relaxed);
+    t.stamps_capacity = t.stamps ? g_stamps_capacity.load(std::memory_order_relaxed) : 0;
+  }
   const int64_t cols = backward ? a.K : a.N;
   const SplitPlan plan = plan_split(a.M, cols, R, grouped);
   const bool split = plan.ksplit > 1 && a.epilogue == EPI_NONE && a.workspace && a.workspace_bytes >= plan.bytes &&
@@ -902,16 +925,13 @@ int splitk_reduce(const float *partial, int parts, int64_t n, void *y, int y_dty
   return launch_status();
 }
 
-int mfma_forward(const GemmArgs &a, hipStream_t s)
-{
-#ifdef CAIFX_DEV
-  const char *sw = getenv("CAIFX_REGW");
-  if (sw && sw[0] == '0') return run(a, false, s);
-#endif
-  const int st = mfma_regw_forward(a, s);
-  return st == CAIFX_ERR_UNSUPPORTED ? run(a, false, s) : st;
-}
+int mfma_tiled_forward(const GemmArgs &a, hipStream_t s) { return run(a, false, s); }
 int mfma_backward(const GemmArgs &a, hipStream_t s) { return run(a, true, s); }
+void mfma_grouped_tile_stamps(void *buf, int64_t tiles)
+{
+  g_stamps_capacity.store(buf ? tiles : 0, std::memory_order_relaxed);
+  g_stamps.store(static_cast<unsigned long long *>(buf), std::memory_order_relaxed);
+}
 size_t mfma_workspace_bytes(const GemmArgs &a, bool backward)
 {
   if (a.compute_dtype == CAIFX_F32) return 0;

@@ -439,4 +439,14 @@ int mfma_regw_forward(const GemmArgs &a, hipStream_t s)
   return launch<f16_t, 4>(t, s);
 }
 
+int mfma_forward(const GemmArgs &a, hipStream_t s)
+{
+#ifdef CAIFX_DEV
+  if (const char *sw = getenv("CAIFX_REGW"))
+    if (sw[0] == '0') return mfma_tiled_forward(a, s);
+#endif
+  const int st = mfma_regw_forward(a, s);
+  return st == CAIFX_ERR_UNSUPPORTED ? mfma_tiled_forward(a, s) : st;
+}
+
 }  // namespace caifx

@@ -520,7 +520,10 @@ __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
 }
 
 // Token-sorted expert segments with few rows each (MoE decode): blockIdx.y is the expert, whose weight is streamed
-// once per 16 rows of its segment; an expert without rows costs nothing.
+// once per 16 rows of its segment; an expert without rows costs nothing.  The host only knows the total row
+// count, so routing may hand one expert most of the rows: the 16-row passes of a segment are dealt out over
+// blockIdx.z, and a long segment is worked on by gridDim.z times as many workgroups instead of gridDim.z times
+// as long (its weight then comes from L2 after the first pass).
 struct MbGroup {
   const int32_t *offsets;
   const void *const *wq_ptrs;
@@ -537,8 +540,9 @@ __global__ __launch_bounds__(kMbThreads) void mblock_grouped_kernel(MbArgs a, Mb
   const uint8_t *wq = static_cast<const uint8_t *>(g.wq_ptrs[e]);
   const void *scales = g.scales_ptrs ? g.scales_ptrs[e] : nullptr;
   const size_t ybytes = a.y_dtype == CAIFX_F32 ? 4 : 2;
-  for (int r = lo; r < hi; r += 16) {
-    if (r > lo) __syncthreads();      // the pass before has read its staging buffers
+  const int first = lo + 16 * static_cast<int>(blockIdx.z);
+  for (int r = first; r < hi; r += 16 * static_cast<int>(gridDim.z)) {
+    if (r > first) __syncthreads();      // the pass before has read its staging buffers
     mblock_body<CT, XT, kInt4, GPW, false>(a, wq, scales, static_cast<const XT *>(a.x) + static_cast<int64_t>(r) * a.K,
                                            static_cast<char *>(a.y) + static_cast<int64_t>(r) * a.N * ybytes,
                                            hi - r < 16 ? hi - r : 16, 0);
@@ -582,7 +586,10 @@ int launch_gpw(const MbArgs &m, size_t lds, hipStream_t s)
 template <typename CT, typename XT, bool kInt4>
 int launch_grouped_gpw(const MbArgs &m, const MbGroup &g, int experts, size_t lds, hipStream_t s)
 {
-  const dim3 grid(static_cast<unsigned>(m.blocks_per_class * m.V), static_cast<unsigned>(experts));
+  // up to eight passes of a segment side by side: with every row in one expert a segment has g.total_rows / 16 passes
+  const int64_t passes = (g.total_rows + 15) / 16;
+  const dim3 grid(static_cast<unsigned>(m.blocks_per_class * m.V), static_cast<unsigned>(experts),
+                  static_cast<unsigned>(passes < 8 ? (passes < 1 ? 1 : passes) : 8));
   const int gpw = (m.groups + kMbWaves - 1) / kMbWaves;
   if (gpw <= 1) hipLaunchKernelGGL((mblock_grouped_kernel<CT, XT, kInt4, 1>), grid, dim3(kMbThreads), lds, s, m, g);
   else if (gpw <= 2) hipLaunchKernelGGL((mblock_grouped_kernel<CT, XT, kInt4, 2>), grid, dim3(kMbThreads), lds, s, m, g);

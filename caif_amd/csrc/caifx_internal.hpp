@@ -61,13 +61,20 @@ size_t mblock_workspace_bytes(const GemmArgs &a);
 int dxrows_backward(const GemmArgs &a, hipStream_t s);
 size_t dxrows_workspace_bytes(const GemmArgs &a);
 
-// Large-M MFMA path (compute bound), forward and input gradient, plain and grouped.
+// Large-M MFMA path (compute bound), forward and input gradient, plain and grouped.  mfma_forward picks between
+// the forward kernels (mfma_regw_forward where it applies, else mfma_tiled_forward).
 int mfma_forward(const GemmArgs &a, hipStream_t s);
+int mfma_tiled_forward(const GemmArgs &a, hipStream_t s);
 int mfma_backward(const GemmArgs &a, hipStream_t s);
 size_t mfma_workspace_bytes(const GemmArgs &a, bool backward);
+// Measurement only: grouped launches of the matrix-core GEMM issued after this call record, per tile of their own
+// numbering (expert by expert, row tile by row tile, column tile last), four 64-bit words {expert, rows in the
+// tile, start, end} with the times in ticks of the 100 MHz wall clock, into buf (device memory for `tiles` tiles);
+// a null buf switches the recording off.  Process-wide.
+void mfma_grouped_tile_stamps(void *buf, int64_t tiles);
 // Forward for packed int4 weights and 16-bit activations of the compute type with enough 128 x 256 tiles to fill
 // the chip: the weight goes from global memory straight into matrix-core operand registers.
-// CAIFX_ERR_UNSUPPORTED for everything else (mfma_forward tries it first).
+// CAIFX_ERR_UNSUPPORTED for everything else.
 int mfma_regw_forward(const GemmArgs &a, hipStream_t s);
 
 // fp32 compute type on the matrix cores (v_mfma_f32_32x32x2_f32), forward and input gradient, any M, plain

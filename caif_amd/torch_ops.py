@@ -146,6 +146,20 @@ def qlinear_forward(x, fw, compute_dtype, y_dtype=F32, out=None, workspace=None,
     return y
 
 
+def probe_mfma_bf16(a_values, b_values, iters):
+    """caifx_probe_mfma_bf16: launches the matrix-pipe-only loop on the first 16384 bf16 values of each tensor;
+    returns the floating-point operations of the launch (time it with events around the call)."""
+    import ctypes
+    _need_cuda(a_values)
+    a = a_values.reshape(-1)[:16384].to(torch.bfloat16).contiguous()
+    b = b_values.reshape(-1)[:16384].to(torch.bfloat16).contiguous()
+    assert a.numel() == 16384 and b.numel() == 16384
+    sink = torch.empty(512, dtype=torch.float32, device=a.device)
+    flops = ctypes.c_int64(0)
+    capi.call("caifx_probe_mfma_bf16", _ptr(a), _ptr(b), int(iters), _ptr(sink), ctypes.byref(flops), _stream())
+    return flops.value, (a, b, sink)
+
+
 def qlinear_backward_input(dy, fw, compute_dtype, dx_dtype=F32, out=None, workspace=None, addend=None):
     """caifx_qlinear_backward_input on dy [..., N]; returns dx [M, K] (plus `addend` [M, K], see qlinear_forward)."""
     _need_cuda(dy)

@@ -213,6 +213,25 @@ CAIFX_API int caifx_qlinear_forward_static(int64_t M, int64_t N, int64_t K,
                                  int group_size,
                                  void *y, int y_dtype, caifx_stream_t stream);
 
+/* Measurement only, no counterpart in the reference (whose per-expert loop, src/caif_device_moe_layer.cpp:534-557,
+ * can simply be timed expert by expert on the host): grouped launches of the matrix-core GEMM issued after this
+ * call record four 64-bit words per tile of 128 rows x 128 columns - {expert, rows of the segment inside the tile,
+ * start, end}, times in ticks of the GPU's 100 MHz wall clock - into `stamps` (device memory for `tiles` tiles, 32
+ * bytes each; tiles are numbered expert by expert, row tile by row tile, column tile last; clear it before a
+ * launch, words of tiles that do not exist stay as they are).  stamps = NULL switches the recording off.
+ * Process-wide state; not meant for timed runs (one more store per workgroup). */
+CAIFX_API int caifx_qlinear_grouped_tile_stamps(void *stamps, int64_t tiles);
+
+/* Measurement only, no counterpart in the reference: `iters` rounds of sixteen v_mfma_f32_32x32x16_bf16 per wave on
+ * every compute unit (eight waves each) over the caller's operand values and nothing else - no loads, no stores,
+ * no unpacking.  a_ops / b_ops: device buffers of 512 * 4 * 8 bf16 values each (16-byte aligned), e.g. a slice of
+ * the activations and of the dequantised weight a benchmark runs on.  The matrix pipes' clock follows the power
+ * the operand bit patterns draw, so this is the ceiling a GEMM on those values is priced against beside the
+ * published peak.  *flops (host, optional) receives the floating-point operations of the launch; sink (device,
+ * optional) 512 floats that keep the compiler from dropping the loop. */
+CAIFX_API int caifx_probe_mfma_bf16(const void *a_ops, const void *b_ops, int64_t iters, void *sink, int64_t *flops,
+                                    caifx_stream_t stream);
+
 /* The per-expert loop of CAIF_DeviceMoELayer over frozen experts
  * (src/caif_device_moe_layer.cpp:534-557 forward, :754-778 backward) as ONE
  * launch: expert e owns rows [offsets[e], offsets[e+1]) of the token-sorted

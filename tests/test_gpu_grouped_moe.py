@@ -135,6 +135,32 @@ def test_grouped_decode_few_rows_per_expert(orc, kind):
     assert compared >= 3
 
 
+@pytest.mark.parametrize("kind", ["int8pc", "int4"])
+def test_grouped_decode_all_rows_in_one_expert(orc, kind):
+    """The host picks the decode kernel from the total row count alone; routing may still send every row to one
+    expert.  16 experts, 250 rows, 243 of them in expert 5 (16 passes of 16 rows, dealt out over the grid's third
+    dimension), a few in two others: every row of every touched expert against the oracle, and the long segment's
+    passes carry the bits of plain calls on their 16 rows."""
+    rng = np.random.default_rng(250)
+    E, N, K = 16, 1408, 2048
+    counts = np.zeros(E, np.int64)
+    counts[5], counts[0], counts[15] = 243, 4, 3
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    total = int(offsets[-1])
+    assert total <= 16 * E
+    ows, gw = _experts(orc, rng, E, N, K, kind)
+    x = dev_as(rng.normal(0, 1, (total, K)), 2)
+    y = T.qlinear_grouped_forward(x, dev(offsets), gw, 2)
+    yh, xh = host(y), host(x)
+    for e in (0, 5, 15):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        assert max_rel_err(yh[lo:hi], orc.frozen_linear_forward(xh[lo:hi], ows[e], 2)) <= TIGHT_POST, (kind, e)
+    lo = int(offsets[5])
+    for p in (0, 7, 15):                                              # a first, a middle and the last (3-row) pass
+        a, b = lo + 16 * p, min(lo + 16 * p + 16, int(offsets[6]))
+        assert torch.equal(y[a:b], T.qlinear_forward(x[a:b].contiguous(), gw.weights[5], 2)), (kind, p)
+
+
 def test_grouped_more_experts_than_lanes(orc):
     # 70 experts: the tile -> expert search runs over more than one 64-lane chunk of the offsets
     rng = np.random.default_rng(12)
