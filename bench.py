@@ -470,6 +470,35 @@ def compute_bound_rows(torch, T, dev, gen, capture, time_graph):
             del g
             rows["lora_base_fwd_bwd_M4096_N11008_K4096"] = {
                 "gemm_cast_add_chain_us": round(ms_c * 1e3, 1), "fused_store_us": round(ms_u * 1e3, 1)}
+    # float-storage cell on the 16-bit matrix cores: weight stored in bf16, bf16 compute (what the reference's bf16
+    # add-MoE runs, CHANGES.md:132-135), forward and input gradient, beside the vendor GEMM on the same operands
+    try:
+        M, N, K = 2048, 4096, 4096
+        wd = torch.empty(N, K, device=dev).normal_(0, 0.02, generator=gen).to(torch.bfloat16)
+        fw = T.FrozenWeight(wd.reshape(-1), T.W_BF16, None, N, K)
+        x = torch.empty(M, K, device=dev).normal_(0, 1, generator=gen).to(torch.bfloat16)
+        dy = torch.empty(M, N, device=dev).normal_(0, 1e-3, generator=gen).to(torch.bfloat16)
+        y, dx = torch.empty(M, N, device=dev), torch.empty(M, K, device=dev)
+        yv = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+        ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+        flops = 2.0 * M * N * K
+        g = capture(lambda i: T.qlinear_forward(x, fw, T.BF16, T.F32, out=y, workspace=ws), L)
+        ms_f = time_graph(g, L, reps=3)
+        del g
+        g = capture(lambda i: T.qlinear_backward_input(dy, fw, T.BF16, T.F32, out=dx, workspace=ws), L)
+        ms_b = time_graph(g, L, reps=3)
+        del g
+        g = capture(lambda i: torch.matmul(x, wd.t(), out=yv), L)
+        ms_v = time_graph(g, L, reps=3)
+        del g
+        rows[f"bf16_storage_M{M}_N{N}_K{K}"] = {
+            "fwd_us": round(ms_f * 1e3, 2), "fwd_TFLOPs": round(flops / (ms_f * 1e-3) / 1e12, 1),
+            "dx_us": round(ms_b * 1e3, 2), "dx_TFLOPs": round(flops / (ms_b * 1e-3) / 1e12, 1),
+            "vendor_dense_bf16_fwd_TFLOPs": round(flops / (ms_v * 1e-3) / 1e12, 1),
+            "fwd_frac_of_vendor": round(ms_v / ms_f, 4)}
+        del wd, fw, x, dy, y, dx, yv
+    except Exception as e:
+        rows["bf16_storage_error"] = repr(e)
     return {"prefill_gemm": rows, "few_tile_gemm": few_tile_rows(torch, T, dev, gen, capture, time_graph),
             "fp32_compute": fp32_rows(torch, T, dev, gen, capture, time_graph),
             "moe_frozen_experts": moe_rows(torch, T, dev, gen)}

@@ -29,6 +29,11 @@ void *static_scratch_on_current_device()
 }
 
 bool float_kind(int w_kind) { return w_kind == CAIFX_W_F32 || w_kind == CAIFX_W_F16 || w_kind == CAIFX_W_BF16; }
+// float storage in the 16-bit compute type itself: the weight needs no conversion and runs on the 16-bit matrix cores
+bool same_16bit(int w_kind, int compute_dtype)
+{
+  return (w_kind == CAIFX_W_BF16 && compute_dtype == CAIFX_BF16) || (w_kind == CAIFX_W_F16 && compute_dtype == CAIFX_F16);
+}
 
 int validate_weight(int64_t N, int64_t K, int w_kind, const void *scales, int64_t scale_period, int group_size)
 {
@@ -112,7 +117,10 @@ size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtyp
   a.compute_dtype = compute_dtype;
   a.w.kind = w_kind;
   const size_t f32_bytes = mfma_f32_workspace_bytes(a, backward != 0);
+  // float storage runs on the fp32 matrix-core kernel unless it is stored in the 16-bit compute type itself
+  if (float_kind(w_kind) && !same_16bit(w_kind, compute_dtype)) return f32_bytes;
   size_t bytes = mfma_workspace_bytes(a, backward != 0);
+  if (float_kind(w_kind)) return f32_bytes > bytes ? f32_bytes : bytes;
   const size_t decode_bytes = backward ? dxrows_workspace_bytes(a) : mblock_workspace_bytes(a);
   if (decode_bytes > bytes) bytes = decode_bytes;
   return f32_bytes > bytes ? f32_bytes : bytes;
@@ -141,7 +149,15 @@ static int forward_impl(int64_t M, int64_t N, int64_t K, const void *x, int x_dt
   GemmArgs a = make_args(M, N, K, x, x_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size, y,
                          y_dtype, workspace, workspace_bytes);
   hipStream_t s = as_stream(stream);
-  if (float_kind(w_kind)) {      // float storage: the fp32 matrix-core kernel, else the shape-agnostic one
+  if (float_kind(w_kind)) {
+    // float storage: stored in the 16-bit compute type -> the tiled kernel on the 16-bit matrix cores; every other
+    // cell the fp32 matrix-core kernel, else the shape-agnostic one
+    if (same_16bit(w_kind, compute_dtype)) {
+      a.addend = addend;
+      st = mfma_forward(a, s);
+      if (st != CAIFX_ERR_UNSUPPORTED) return st;       // added in the store
+      a.addend = nullptr;
+    }
     st = mfma_f32_forward(a, s);
     if (st == CAIFX_ERR_UNSUPPORTED) st = generic_forward(a, s);
     return finish_add(st, addend, y, y_dtype, M * N, stream);
@@ -252,6 +268,12 @@ static int backward_impl(int64_t M, int64_t N, int64_t K, const void *dy, int dy
     st = dxrows_backward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, dx, dx_dtype, M * K, stream);
   }
+  if (same_16bit(w_kind, compute_dtype)) {
+    a.addend = addend;
+    st = mfma_backward(a, s);
+    if (st != CAIFX_ERR_UNSUPPORTED) return st;         // added in the store
+    a.addend = nullptr;
+  }
   if (compute_dtype == CAIFX_F32 || float_kind(w_kind)) {
     st = mfma_f32_backward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, dx, dx_dtype, M * K, stream);
@@ -326,6 +348,12 @@ static int grouped(bool backward, int num_experts, const int32_t *offsets, int64
   a.num_experts = num_experts;
   if (addend && (addend == y || !aligned_to(addend, dtype_size(y_dtype)))) return CAIFX_ERR_INVALID_ARGUMENT;
   hipStream_t s = as_stream(stream);
+  if (same_16bit(w_kind, compute_dtype)) {
+    a.addend = addend;
+    st = backward ? mfma_backward(a, s) : mfma_forward(a, s);
+    if (st != CAIFX_ERR_UNSUPPORTED) return st;
+    a.addend = nullptr;
+  }
   if ((compute_dtype == CAIFX_F32 || float_kind(w_kind)) && !addend) {
     st = backward ? mfma_f32_backward(a, s) : mfma_f32_forward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return st;

@@ -39,6 +39,30 @@ def test_float_storage_forward_backward(orc, sd, cd, M, N, K):
     assert max_rel_err(dx, orc.frozen_linear_backward(host(dy), ow, cd)) <= bound
 
 
+@pytest.mark.parametrize("sd", [1, 2])
+@pytest.mark.parametrize("M,N,K", [(2048, 1024, 512),      # full 256-row tiles forward, 128-row tiles for the gradient
+                                   (300, 1100, 1408),      # ragged rows and columns; the gradient reduces over 1100: other kernel
+                                   (64, 2048, 2048)])      # few tiles: workgroups share each tile's reduction
+def test_same_type_16bit_storage_on_the_16bit_matrix_cores(orc, sd, M, N, K):
+    # weight stored in the compute type (bf16 / bf16, fp16 / fp16): the tiled kernel with the dequantisation compiled
+    # out, src/caif_device_frozen_linear.cpp:301-318 (same-dtype view) + :465-509; fp32 and storage-type results,
+    # and the fused Add of a LoRA-style branch
+    rng = np.random.default_rng(1000 * sd + M)
+    ow, dw = _weight(orc, rng, N, K, sd)
+    x = dev_as(rng.normal(0, 1, (M, K)), sd)
+    dy = dev_as(rng.normal(0, 1e-2, (M, N)), sd)
+    sel = np.sort(rng.choice(M, min(M, 24), replace=False))
+    y = T.qlinear_forward(x, dw, sd)
+    assert max_rel_err(host(y)[sel], orc.frozen_linear_forward(host(x)[sel], ow, sd)) <= 2e-5
+    dx = T.qlinear_backward_input(dy, dw, sd)
+    assert max_rel_err(host(dx)[sel], orc.frozen_linear_backward(host(dy)[sel], ow, sd)) <= 2e-5
+    y16 = T.qlinear_forward(x, dw, sd, sd)
+    assert torch.equal(y16, y.to(TORCH_OF[sd]))
+    add = dev_as(rng.normal(0, 1, (M, N)), sd)
+    fused = T.qlinear_forward(x, dw, sd, sd, addend=add)
+    assert torch.equal(fused, (y16.float() + add.float()).to(TORCH_OF[sd]))
+
+
 def test_float_storage_fp32_is_the_dense_product(orc):
     # storage and compute both fp32: the layout pin of tests/test_device_frozen_linear.cpp:996-1072
     # (W is [output_dim, input_dim], y = x W^T) against torch's own GEMM
