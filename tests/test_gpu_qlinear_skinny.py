@@ -352,10 +352,11 @@ def test_input_gradient_few_rows_other_paths(orc):
     _check_dx(orc, rng, 3, 40, 128, "int8pt", 0, 0, workspace=none)     # one workgroup: no workspace needed
 
 
-@pytest.mark.parametrize("N,K,M", [(1536, 1024, 16), (14336, 4096, 4), (3584, 1024, 9)])
+@pytest.mark.parametrize("N,K,M", [(1536, 1024, 16), (14336, 4096, 4), (14336, 4096, 16), (3584, 1024, 9)])
 def test_input_gradient_few_rows_residue_classes(orc, N, K, M):
     # one scale per output feature with K mod N != 0: the scale of W[n][k] depends on n, but rows with equal
-    # n mod V (V = 3, 7, 7 here) share their scales along k; a workgroup stays inside one class
+    # n mod V (V = 3, 7, 7, 7 here) share their scales along k; a workgroup stays inside one class.  (14336, 4096) is
+    # BASELINE configs[1]'s up projection at full width, with 4 rows and with all 16.
     rng = np.random.default_rng(N + K + M)
     assert _check_dx(orc, rng, M, N, K, "int8pc", 0, 0) <= 2e-6
     assert _check_dx(orc, rng, M, N, K, "int8pc", 2, 2) <= TIGHT_POST

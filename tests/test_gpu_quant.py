@@ -72,6 +72,27 @@ def test_int4_bit_exact(orc, n, group):
     assert np.array_equal(host(d).view(np.uint32), orc.dequantize_int4(po, so, n, group).view(np.uint32))
 
 
+def test_quantisers_at_the_decode_weight_bit_exact(orc):
+    """BASELINE configs[1]'s weight at its real size against the oracle, bit for bit: per-channel int8 on the
+    [4096, 14336] buffer the reference labels [in, out] (src/caif_cuda_kernels_quant.cu:488-558; 14336 column
+    maxima, seven residue classes of column phase per 16-byte lane) and int4 with groups of 128 on its 58,720,256
+    elements (:281-330; 458,752 groups)."""
+    rng = np.random.default_rng(14336)
+    K, N = 4096, 14336
+    w = rng.normal(0, 0.02, (K, N)).astype(np.float32)
+    w[rng.integers(0, K, 2000), rng.integers(0, N, 2000)] = 0.0
+    wd = dev(w)
+    q, s = T.quantize_int8(wd, per_channel=True)
+    qo, so = orc.quantize_int8_per_channel(w)
+    assert np.array_equal(host(s).view(np.uint32), so.view(np.uint32))
+    assert np.array_equal(host(q), qo)
+    del q, s, qo, so
+    p, s4 = T.quantize_int4_per_group(wd.reshape(-1), 128)
+    po, so4 = orc.quantize_to_int4(w.reshape(-1), 128)
+    assert np.array_equal(f16_bits(s4), so4)
+    assert np.array_equal(host(p), po)
+
+
 def test_int4_decodes_code_minus_eight(orc):
     rng = np.random.default_rng(3)
     packed = rng.integers(0, 256, 4096, dtype=np.uint8)         # every nibble value incl. 0x8
