@@ -29,7 +29,10 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 MFMA_FP32_PEAK_TFLOPS = 157.3
 K_DEC, N_DEC = 4096, 14336
-MEASURED_TRAFFIC_INT8_M1 = 59406822     # bytes per launch, rocprofv3 counters (see the roofline object)
+# HBM bytes per launch of the dominant kernel from rocprofv3 counters (profiles/decode_gemv_hbm_traffic.md).  A counter run
+# cannot happen inside this script, so the figure is carried here with the state of the tree it was collected on.
+MEASURED_TRAFFIC_INT8_M1 = 59406822
+MEASURED_TRAFFIC_COLLECTED = "commit a3f0718 (after the last change to rowlin_int8_digits_kernel); same readings as the first collection"
 
 
 def algorithmic_bytes(kind, M, N=N_DEC, K=K_DEC, group=128):
@@ -181,6 +184,7 @@ def main():
         # WRITE_SIZE x 1.0000, factors from a plain 256 MiB copy in the same runs): 59.35 MB read +
         # 0.06 MB written; the summary is profiles/decode_gemv_hbm_traffic.md
         "traffic": MEASURED_TRAFFIC_INT8_M1,
+        "traffic_collected_at": MEASURED_TRAFFIC_COLLECTED,
     }
 
     extra = {
@@ -260,14 +264,12 @@ def decode_other_rows(torch, T, dev, gen, capture, time_graph):
                                        "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                        "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     # yardstick, not part of the path: what kernels that are not this library's read per second from the same
-    # rotated buffers (each launch a different 470 MB copy, so nothing comes from cache): a sum over the bytes
-    # (one pass of reads, nothing written) and a device-to-device copy (half reads, half writes)
+    # rotated buffers (each launch a different 470 MB copy, so nothing comes from cache): the runtime's device-to-device
+    # copy, half reads, half writes (torch's reductions run far below the memory rate and say nothing here)
     try:
         bufs = [fw.wq for fw in tall[1][1]]
         nb = bufs[0].numel()
-        views = [b.view(torch.int32) for b in bufs]
         sink = torch.empty(nb, dtype=torch.int8, device=dev)
-        acc = torch.zeros((), dtype=torch.int64, device=dev)
 
         def timed(fn, n=6):
             fn(0)
@@ -280,11 +282,9 @@ def decode_other_rows(torch, T, dev, gen, capture, time_graph):
             torch.cuda.synchronize()
             return e0.elapsed_time(e1) / n
 
-        ms_sum = timed(lambda i: acc.copy_(views[i % len(views)].sum(dtype=torch.int64)))
         ms_cpy = timed(lambda i: sink.copy_(bufs[i % len(bufs)]))
-        out["hbm_stream_yardstick_GBps"] = {"bytes": nb, "torch_sum_read_only": round(nb / (ms_sum * 1e-3) / 1e9, 1),
-                                            "device_copy_read_plus_write": round(2 * nb / (ms_cpy * 1e-3) / 1e9, 1)}
-        del bufs, views, sink, acc
+        out["hbm_stream_yardstick_GBps"] = {"bytes": nb, "device_copy_read_plus_write": round(2 * nb / (ms_cpy * 1e-3) / 1e9, 1)}
+        del bufs, sink
     except Exception as e:   # a yardstick must not take the rows down
         out["hbm_stream_yardstick_GBps"] = None
         print(f"bench: HBM stream yardstick skipped: {type(e).__name__}: {e}", file=sys.stderr)
