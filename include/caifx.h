@@ -190,8 +190,14 @@ CAIFX_API int caifx_qlinear_backward_input_add(int64_t M, int64_t N, int64_t K,
  * to 16 rows, K > 2048 with 17..32 rows or with int8 codes and N small enough that the activations' preparation
  * outweighs a workgroup's share of the weight), and the input gradient with up to 16 rows splits
  * the weight's rows among workgroups the same way.  With a smaller or null
- * workspace the calls run without that sharing, only slower, and the sums are formed in a different order, so
- * the last bits of a result may differ between a call with and a call without the workspace. */
+ * workspace the calls run without that sharing, slower, and the sums are formed in a different order, so
+ * the last bits of a result differ between a call with and a call without the workspace.  In two places the
+ * workspace also selects between the two accuracy classes of caifx_qlinear_forward's comment: the input gradient
+ * with up to 16 rows and the forward with up to 16 rows and K > 4096 run, without it, on kernels that round
+ * code * scale to the 16-bit compute type as the reference does, and with it on the few-row kernels that multiply
+ * unrounded codes (about 2e-3 of max|out| apart; both within the 1e-2 bound).  Packed int4 with a 16-bit compute
+ * type is the other way round for the input gradient: with the workspace it takes the tiled kernel (rounded
+ * weight), without it the few-row kernel when that needs no workspace. */
 CAIFX_API size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtype, int compute_dtype,
                                      int w_kind, int backward);
 
