@@ -24,7 +24,7 @@ EXPORTS = [
     "caifx_quantize_int8_per_channel", "caifx_dequantize_int8_per_channel",
     "caifx_quantize_to_int4", "caifx_dequantize_int4",
     "caifx_qlinear_forward", "caifx_qlinear_backward_input", "caifx_qlinear_workspace_bytes",
-    "caifx_qlinear_forward_static", "caifx_probe_mfma_bf16", "caifx_qlinear_grouped_tile_stamps",
+    "caifx_qlinear_forward_static", "caifx_static_scratch_prepare", "caifx_probe_mfma_bf16", "caifx_qlinear_grouped_tile_stamps",
     "caifx_qlinear_forward_add", "caifx_qlinear_backward_input_add", "caifx_qlinear_grouped_backward_input_add",
     "caifx_qlinear_grouped_forward", "caifx_qlinear_grouped_backward_input",
     "caifx_qlinear_grouped_workspace_bytes", "caifx_qlinear_grouped_forward_swiglu",
@@ -80,6 +80,7 @@ def lib():
         L.caifx_qlinear_backward_input.argtypes = gemm
         L.caifx_qlinear_forward_static.argtypes = gemm[:13] + [_p]      # no workspace pair
         L.caifx_qlinear_grouped_tile_stamps.argtypes = [_p, _i64]
+        L.caifx_static_scratch_prepare.argtypes = []
         L.caifx_probe_mfma_bf16.argtypes = [_p, _p, _i64, _p, ctypes.POINTER(ctypes.c_int64), _p]
         gemm_add = gemm[:13] + [_p] + gemm[13:]                     # addend after (y, y_dtype)
         L.caifx_qlinear_forward_add.argtypes = gemm_add

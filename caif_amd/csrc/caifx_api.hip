@@ -220,6 +220,16 @@ int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K, const void *x, int x_
                       nullptr, workspace, workspace_bytes, stream);
 }
 
+int caifx_static_scratch_prepare(void)
+{
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return CAIFX_ERR_LAUNCH_FAILED;
+  void *p = nullptr;
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch)) != hipSuccess || !p) return CAIFX_ERR_LAUNCH_FAILED;
+  static_scratch_ptr[dev].store(p, std::memory_order_release);       // also replaces an address from before a device reset
+  return CAIFX_OK;
+}
+
 int caifx_qlinear_forward_static(int64_t M, int64_t N, int64_t K, const void *x, int x_dtype, int compute_dtype,
                                  const void *wq, int w_kind, const void *scales, int64_t scale_period, int group_size,
                                  void *y, int y_dtype, caifx_stream_t stream)

@@ -185,17 +185,18 @@ class CAIF_DeviceFrozenLinear:public CAIF_DeviceLayerTyped<ComputeT,StorageT>,
       {
         if(index!=0){THROW_CAIFE("FrozenLinear: frozen tensor index out of range");}
         if(_weight.IsEmpty()==true){THROW_CAIFE("FrozenLinear: weight not loaded");}
-        const int64_t total=static_cast<int64_t>(InputDim())*OutputDim();
-        CAIF_DeviceTensor fp32=CAIF_DeviceTensor::Uninitialized({OutputDim(),InputDim()},Stream());
-        hipStream_t s=Stream().Handle();
-        int st;
         if(IsFloatStorage()==true)
         {
-          // float storage: the weight itself, widened (src/caif_device_frozen_linear.cpp:780-790)
+          // float storage: the weight itself, widened (src/caif_device_frozen_linear.cpp:780-790); nothing else is
+          // allocated on this path
           CAIF_DeviceTensor wide=_weight.To(Dtype_e::Float32);
           wide.Reshape({OutputDim(),InputDim()});
           return wide;
         }
+        const int64_t total=static_cast<int64_t>(InputDim())*OutputDim();
+        CAIF_DeviceTensor fp32=CAIF_DeviceTensor::Uninitialized({OutputDim(),InputDim()},Stream());
+        hipStream_t s=Stream().Handle();
+        int st;
         if(IsInt4()==true)
         {
           if(_scales.IsEmpty()==true){THROW_CAIFE("FrozenLinear: scales not loaded");}

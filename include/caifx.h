@@ -211,8 +211,13 @@ CAIFX_API size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, 
  * launches nothing (use caifx_qlinear_forward then; with a null workspace it runs without sharing).
  * The call itself allocates and frees nothing.  Every call on one GPU uses that GPU's one buffer: calls on
  * different streams of the same GPU that may overlap race on it; calls on one stream are ordered and need no
- * clearing in between (every partial tile is written in full before it is read). */
+ * clearing in between (every partial tile is written in full before it is read).
+ * The buffer's address on a GPU is looked up (hipGetSymbolAddress) on the first call there and kept for the life
+ * of the process.  A caller that captures the call into a HIP graph should have that lookup done before the
+ * capture begins, by an earlier call or by caifx_static_scratch_prepare() with that GPU current (which also
+ * refreshes the address after a hipDeviceReset). */
 #define CAIFX_STATIC_SCRATCH_BYTES (8u << 20)
+CAIFX_API int caifx_static_scratch_prepare(void);
 CAIFX_API int caifx_qlinear_forward_static(int64_t M, int64_t N, int64_t K,
                                  const void *x, int x_dtype, int compute_dtype,
                                  const void *wq, int w_kind, const void *scales, int64_t scale_period,
