@@ -647,7 +647,7 @@ def moe_rows(torch, T, dev, gen):
     # Per-expert-segment GEMM efficiency (outside the timed runs): the grouped kernel stamps every 128 x 128 tile
     # with its expert, row count, start and end (100 MHz wall clock).  An expert's efficiency is the flops of its
     # segment over what the matrix pipes offer during its tiles' lifetimes, 2 cnt K N / (sum of tile durations x
-    # peak / (256 compute units x 2 workgroups that share one)); partial last tiles and everything a tile waits
+    # peak / (256 compute units x the workgroups that share one)); partial last tiles and everything a tile waits
     # for count against it.
     def segment_efficiency(launch, n_cols, k_red):
         from caif_amd import capi
@@ -662,7 +662,10 @@ def moe_rows(torch, T, dev, gen):
         st = stamps.view(-1, 4).cpu()
         st = st[st[:, 3] > 0]
         cnt = counts.cpu()
-        share = MFMA_BF16_PEAK_TFLOPS * 1e12 / (256 * 2)
+        # word 1 of a stamp: rows of the tile, and from bit 32 up how many workgroups of the kernel that ran it
+        # share a compute unit when that is not two (the int8 forward kernel runs one)
+        resident = int(st[0, 1] >> 32) or 2
+        share = MFMA_BF16_PEAK_TFLOPS * 1e12 / (256 * resident)
         effs = []
         for e in range(E):
             mine = st[st[:, 0] == e]
@@ -672,11 +675,11 @@ def moe_rows(torch, T, dev, gen):
             effs.append(2.0 * int(cnt[e]) * n_cols * k_red / (busy_s * share))
         effs.sort()
         span_s = float(st[:, 3].max() - st[:, 2].min()) / 1e8
-        return {"experts": len(effs), "tiles": int(len(st)), "min": round(effs[0], 4), "median": round(effs[len(effs) // 2], 4),
+        return {"experts": len(effs), "tiles": int(len(st)), "workgroups_per_cu": resident, "min": round(effs[0], 4), "median": round(effs[len(effs) // 2], 4),
                 "max": round(effs[-1], 4), "first_start_to_last_end_us": round(span_s * 1e6, 1)}
 
     try:
-        seg = {"definition": "2*rows_e*K*N / (sum of the expert's tile durations * 2.5 PFLOP/s / 512 resident workgroups)",
+        seg = {"definition": "2*rows_e*K*N / (sum of the expert's tile durations * 2.5 PFLOP/s / (256 * workgroups_per_cu))",
                "gate_forward_2048_to_1408": segment_efficiency(
                    lambda: T.qlinear_grouped_forward(x, offsets, gate, T.BF16, T.BF16, out=gate_o, workspace=ws), H, D),
                "down_forward_1408_to_2048": segment_efficiency(

@@ -1,5 +1,6 @@
 // Host side of the tiled dequant-GEMM for integer codes (int8, packed int4): argument checks, tile and
 // scale-mode choice, the shared reduction for launches with few tiles.  The kernel is in caifx_gemm_tile.hpp.
+#include "caifx_gemm_regw.hpp"
 #include "caifx_gemm_tile.hpp"
 
 #include <cstdlib>
@@ -185,6 +186,12 @@ int splitk_reduce(const float *partial, int parts, int64_t n, void *y, int y_dty
 
 int mfma_tiled_forward(const GemmArgs &a, hipStream_t s) { return run(a, false, s); }
 int mfma_backward(const GemmArgs &a, hipStream_t s) { return run(a, true, s); }
+void mfma_grouped_stamp_target(unsigned long long **buf, long long *capacity)
+{
+  *buf = g_stamps.load(std::memory_order_relaxed);
+  *capacity = *buf ? g_stamps_capacity.load(std::memory_order_relaxed) : 0;
+}
+
 void mfma_grouped_tile_stamps(void *buf, int64_t tiles)
 {
   g_stamps_capacity.store(buf ? tiles : 0, std::memory_order_relaxed);

@@ -29,7 +29,7 @@
 // untouched between its request and the hand-placed wait, which the compiler does not promise.
 // The store goes through LDS as a whole tile so that one wave instruction writes one contiguous row piece of the
 // tile (1 KiB of fp32) instead of eight 128-byte pieces.
-#include "caifx_internal.hpp"
+#include "caifx_gemm_regw.hpp"
 
 #include <atomic>
 #include <cstdlib>
@@ -38,9 +38,10 @@
 namespace caifx {
 namespace {
 
-constexpr int kBK = 64;        // reduction extent of a step
-constexpr int kBN = 256;       // columns of Y per workgroup: 8 waves x 32
-constexpr int kStages = 4;     // LDS ring of activation tiles
+using regw::kBK;
+using regw::kBN;
+using regw::kStages;
+using regw::swz;
 constexpr int kWAhead = 7;     // code request u (8 weight rows x 256 codes: rows 8 (u % 4) .., block u / 4) is issued in step u - 7
 constexpr int kWSlots = 10;    // ... into slot u % 10 of the wave's ring
 constexpr int kGroup = 128;    // int4 group size this kernel is written for: one scale dword per weight row and block
@@ -54,9 +55,6 @@ struct RegwArgs {
   const uint8_t *wq;
   const f16_t *scales;
 };
-
-// byte offset of 16-byte chunk `chunk` (0..7) of row `row` in an LDS tile of 128-byte rows
-__device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + ((chunk ^ ((row ^ (row >> 3)) & 7)) << 4); }
 
 // eight int4 codes of one dword (nibble t = element t) times one scale, rounded to CT: fma(code + 8, s, -8 s) is
 // the exact product float(code) * s (m8 = -8 s and s16 = s / 16 are exact), so the only rounding is the cast.
@@ -317,82 +315,20 @@ __global__ __launch_bounds__(512, 2) void qgemm_regw_kernel(RegwArgs g)
   // requests past the last step may still be writing LDS, and other waves may still be reading
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 
-  // ---- store: acc[i][r] = Y[row0 + 32 i + 8 (r / 4) + 4 (lane / 32) + r % 4][col0 + 32 wave + lane % 32].
-  // The whole tile is laid out in LDS (row pitch = row + 32 bytes, so the two lane halves, four rows apart, use
-  // different halves of the banks), then every wave writes whole tile rows: 16 bytes per lane, 1 KiB (fp32) or two
-  // rows of 512 bytes (16-bit results) per instruction, and reads the optional addend the same way.  Tiles taller
-  // than the LDS holds go in passes of kPassRows rows.
-  auto store = [&](auto tag) {
-    typedef decltype(tag) T;
-    constexpr int kPitch = kBN * sizeof(T) + 32;
-    constexpr int kPer16 = 16 / sizeof(T);                 // elements per 16-byte piece
-    constexpr int kLanesPerRow = kBN / kPer16;             // 64 (fp32) or 32
-    constexpr int kRowsPerInstr = 64 / kLanesPerRow;       // 1 or 2
-    constexpr int kPassRows = (BM * kPitch <= 150 * 1024) ? BM : BM / 2;
-    constexpr int kPassBlocks = kPassRows / 32;
-    const int chunk = lane % kLanesPerRow;
-    const int64_t gcol = col0 + chunk * kPer16;
-    T *dp = static_cast<T *>(g.d);
-    const T *ap = static_cast<const T *>(g.addend);
-    const bool vec_ok = (g.N % kPer16 == 0);
-#pragma unroll
-    for (int pass = 0; pass < BM / kPassRows; ++pass) {
-      if (pass > 0) __syncthreads();
-#pragma unroll
-      for (int ii = 0; ii < kPassBlocks; ++ii) {
-        const int i = pass * kPassBlocks + ii;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int lrow = ii * 32 + 8 * (r >> 2) + 4 * fh + (r & 3);
-          *reinterpret_cast<T *>(smem + lrow * kPitch + (wave * 32 + frow) * sizeof(T)) = from_f32<T>(acc[i][r]);
-        }
-      }
-      __syncthreads();
-      constexpr int kInstr = kPassRows / (8 * kRowsPerInstr);      // row pieces per wave
-#pragma unroll
-      for (int it = 0; it < kInstr; ++it) {
-        const int lrow = (it * 8 + wave) * kRowsPerInstr + lane / kLanesPerRow;
-        const int64_t grow = row0 + pass * kPassRows + lrow;
-        if (grow >= g.M || gcol >= g.N) continue;
-        u32x4_t v = *reinterpret_cast<const u32x4_t *>(smem + lrow * kPitch + chunk * 16);
-        const int64_t o = grow * g.N + gcol;
-        if (vec_ok) {
-          if (ap) {
-            const u32x4_t av = *reinterpret_cast<const u32x4_t *>(ap + o);
-            const T *vp = reinterpret_cast<const T *>(&v);
-            const T *aq = reinterpret_cast<const T *>(&av);
-            u32x4_t w;
-            T *wp = reinterpret_cast<T *>(&w);
-#pragma unroll
-            for (int e = 0; e < kPer16; ++e) wp[e] = from_f32<T>(to_f32<T>(vp[e]) + to_f32<T>(aq[e]));
-            v = w;
-          }
-          *reinterpret_cast<u32x4_t *>(dp + o) = v;
-        } else {
-          const T *vp = reinterpret_cast<const T *>(&v);
-#pragma unroll
-          for (int e = 0; e < kPer16; ++e) {
-            if (gcol + e < g.N) {
-              T val = vp[e];
-              if (ap) val = from_f32<T>(to_f32<T>(val) + to_f32<T>(ap[o + e]));
-              dp[o + e] = val;
-            }
-          }
-        }
-      }
-    }
-  };
-  if (g.d_dtype == CAIFX_BF16) store(bf16_t{});
-  else if (g.d_dtype == CAIFX_F16) store(f16_t{});
-  else store(float{});
+  // ---- store (regw::store_tile: the whole tile through LDS, whole rows per wave instruction)
+  if (g.d_dtype == CAIFX_BF16)
+    regw::store_tile<bf16_t, WR>(smem, acc, wave, lane, row0, g.M, col0, g.N, static_cast<bf16_t *>(g.d), static_cast<const bf16_t *>(g.addend));
+  else if (g.d_dtype == CAIFX_F16)
+    regw::store_tile<f16_t, WR>(smem, acc, wave, lane, row0, g.M, col0, g.N, static_cast<f16_t *>(g.d), static_cast<const f16_t *>(g.addend));
+  else
+    regw::store_tile<float, WR>(smem, acc, wave, lane, row0, g.M, col0, g.N, static_cast<float *>(g.d), static_cast<const float *>(g.addend));
 }
 
 template <typename CT, int WR> int launch(const RegwArgs &t, hipStream_t s)
 {
   constexpr int BM = 32 * WR;
   const size_t ring = static_cast<size_t>(kStages) * BM * kBK * 2 + 8 * kWSlots * 1024 + 8 * 3 * 256;
-  const size_t pass_rows = static_cast<size_t>(BM) * (kBN * 4 + 32) <= 150 * 1024 ? BM : BM / 2;
-  const size_t staging = pass_rows * (kBN * 4 + 32);
+  const size_t staging = regw::store_bytes(BM);
   const size_t lds = ring > staging ? ring : staging;
   auto kern = qgemm_regw_kernel<CT, WR>;
   static std::atomic<bool> raised{false};
@@ -445,7 +381,8 @@ int mfma_forward(const GemmArgs &a, hipStream_t s)
   if (const char *sw = getenv("CAIFX_REGW"))
     if (sw[0] == '0') return mfma_tiled_forward(a, s);
 #endif
-  const int st = mfma_regw_forward(a, s);
+  int st = mfma_regw_forward(a, s);
+  if (st == CAIFX_ERR_UNSUPPORTED) st = mfma_regw8_forward(a, s);
   return st == CAIFX_ERR_UNSUPPORTED ? mfma_tiled_forward(a, s) : st;
 }
 
