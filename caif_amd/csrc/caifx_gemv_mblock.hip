@@ -146,7 +146,8 @@ constexpr int kSegRows = kSegBlocks * 16;
 // unpacked once and multiplied with each tile's operands.
 // wq / scales: the weight; xrows / yrows: the first of the M activation and result rows; slice: which part of
 // the reduction (see MbArgs).  Every thread of the workgroup makes the same calls (the body has barriers).
-template <typename CT, typename XT, bool kInt4, int GPW, bool kF32, int MT = 1>
+// D: row blocks a wave keeps requested (1 or 2; the launch code picks by measurement)
+template <typename CT, typename XT, bool kInt4, int GPW, bool kF32, int MT = 1, int D = 2>
 __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, const void *scales, const void *xrows,
                                             void *yrows, int M, int slice)
 {
@@ -154,7 +155,6 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
   typedef typename Mfma16<CT>::vec_t vec_t;
   constexpr int LPG = kInt4 ? 1 : 2;           // 16-byte loads per lane per 128-k group
   constexpr int LPR = GPW * LPG;               // ... per block of 16 weight rows
-  constexpr int D = 2;                         // row blocks in the ring
   constexpr int RBB = mb_reduce_blocks(kInt4, MT);      // row blocks between two reductions (a multiple of D, divides kSegBlocks)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float *partial = reinterpret_cast<float *>(smem);      // [RBB][MT][16 waves][4][64]
@@ -513,10 +513,10 @@ __device__ __forceinline__ void mblock_body(const MbArgs &a, const uint8_t *wq, 
   }
 }
 
-template <typename CT, typename XT, bool kInt4, int GPW, bool kF32 = false, int MT = 1>
+template <typename CT, typename XT, bool kInt4, int GPW, bool kF32 = false, int MT = 1, int D = 2>
 __global__ __launch_bounds__(kMbThreads) void mblock_kernel(MbArgs a)
 {
-  mblock_body<CT, XT, kInt4, GPW, kF32, MT>(a, a.wq, a.scales, a.x, a.y, a.M, blockIdx.y);
+  mblock_body<CT, XT, kInt4, GPW, kF32, MT, D>(a, a.wq, a.scales, a.x, a.y, a.M, blockIdx.y);
 }
 
 // Token-sorted expert segments with few rows each (MoE decode): blockIdx.y is the expert, whose weight is streamed
@@ -570,9 +570,20 @@ int launch_gpw(const MbArgs &m, size_t lds, hipStream_t s)
                   static_cast<unsigned>((m.groups + m.slice_groups - 1) / m.slice_groups));
   const int gpw = (m.slice_groups + kMbWaves - 1) / kMbWaves;
   if (m.M <= 16) {
-    if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 1, kF32>), grid, dim3(kMbThreads), lds, s, m);
-    else if (gpw <= 2) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 2, kF32>), grid, dim3(kMbThreads), lds, s, m);
-    else return CAIFX_ERR_UNSUPPORTED;
+    // One row block requested at a time instead of two, by measurement (K = 4096, N = 2048 ... 28672, times in us):
+    // int4 with 4 rows 7.2 -> 6.6, 7.9 -> 7.1, 9.6 -> 9.1, 11.0 -> 10.6, 12.7 -> 12.4, 20.4 -> 19.7; with 16 rows
+    // 9.0 -> 8.4, 9.4 -> 8.9, 11.3 -> 11.2, 12.8 -> 13.1, 14.7 -> 14.9, 23.0 -> 22.4, so two stay only for more than 8
+    // rows with 33..64 weight rows per workgroup; int8 gains up to 32 weight rows per workgroup (10.8 -> 10.6,
+    // 11.5 -> 11.35 at N = 4096) and loses 1.5 us beyond.
+    const int64_t rows_class = (m.N + m.V - 1) / m.V;
+    const int64_t rows_wg = (rows_class + m.blocks_per_class - 1) / m.blocks_per_class;
+    const bool one_block = kInt4 ? (m.M <= 8 || rows_wg <= 32 || rows_wg > 64) : rows_wg <= 32;
+    if (gpw > 2) return CAIFX_ERR_UNSUPPORTED;
+    if (one_block) {
+      if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 1, kF32, 1, 1>), grid, dim3(kMbThreads), lds, s, m);
+      else hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 2, kF32, 1, 1>), grid, dim3(kMbThreads), lds, s, m);
+    } else if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 1, kF32>), grid, dim3(kMbThreads), lds, s, m);
+    else hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 2, kF32>), grid, dim3(kMbThreads), lds, s, m);
   } else {
     if (gpw <= 1) hipLaunchKernelGGL((mblock_kernel<CT, XT, kInt4, 1, kF32, 2>), grid, dim3(kMbThreads), lds, s, m);
     else if constexpr (mb_max_gpw(kInt4, 2) >= 2) {
