@@ -226,10 +226,12 @@ CAIFX_API int caifx_qlinear_forward_static(int64_t M, int64_t N, int64_t K,
 
 /* Measurement only, no counterpart in the reference (whose per-expert loop, src/caif_device_moe_layer.cpp:534-557,
  * can simply be timed expert by expert on the host): grouped launches of the matrix-core GEMM issued after this
- * call record four 64-bit words per tile of 128 rows x 128 columns - {expert, rows of the segment inside the tile,
- * start, end}, times in ticks of the GPU's 100 MHz wall clock - into `stamps` (device memory for `tiles` tiles, 32
- * bytes each; tiles are numbered expert by expert, row tile by row tile, column tile last; clear it before a
- * launch, words of tiles that do not exist stay as they are).  stamps = NULL switches the recording off.
+ * call record four 64-bit words per tile (128 rows x 128 columns, or x 256 for the int8 forward kernel that keeps
+ * the weight out of LDS) - {expert, rows of the segment inside the tile (low 32 bits; from bit 32 up, when not 0,
+ * how many workgroups of that kernel share a compute unit instead of two), start, end}, times in ticks of the
+ * GPU's 100 MHz wall clock - into `stamps` (device memory for `tiles` tiles, 32 bytes each; sizing for 128 x 128
+ * tiles covers both; tiles are numbered expert by expert, row tile by row tile, column tile last; clear it before
+ * a launch, words of tiles that do not exist stay as they are).  stamps = NULL switches the recording off.
  * Process-wide state; not meant for timed runs (one more store per workgroup). */
 CAIFX_API int caifx_qlinear_grouped_tile_stamps(void *stamps, int64_t tiles);
 
