@@ -32,7 +32,7 @@ K_DEC, N_DEC = 4096, 14336
 # HBM bytes per launch of the dominant kernel from rocprofv3 counters (profiles/decode_gemv_hbm_traffic.md).  A counter run
 # cannot happen inside this script, so the figure is carried here with the state of the tree it was collected on.
 MEASURED_TRAFFIC_INT8_M1 = 59406822
-MEASURED_TRAFFIC_COLLECTED = "commit a3f0718 (after the last change to rowlin_int8_digits_kernel); same readings as the first collection"
+MEASURED_TRAFFIC_COLLECTED = "commit a3f0718 (after the last change to rowlin_int8_digits_kernel); read again at commit fdff18f: the same counts"
 
 
 def algorithmic_bytes(kind, M, N=N_DEC, K=K_DEC, group=128):
