@@ -1,6 +1,8 @@
 // extern "C" entry points of the dequant-GEMM seam: argument validation and kernel choice.
 #include "caifx_internal.hpp"
 
+#include <cstdlib>
+
 #include <atomic>
 
 using namespace caifx;
@@ -272,16 +274,13 @@ static int backward_impl(int64_t M, int64_t N, int64_t K, const void *dy, int dy
   GemmArgs a = make_args(M, N, K, dy, dy_dtype, compute_dtype, wq, w_kind, scales, scale_period, group_size,
                          dx, dx_dtype, workspace, workspace_bytes);
   hipStream_t s = as_stream(stream);
-  // up to 16 rows of int8 codes whose scales do not depend on the weight row, or of int4 codes in groups of 128
-  // or more: one pass over the weight at the memory rate, whatever the compute type
-  // Packed int4 with a 16-bit compute type is the exception when the tiled kernel can share each tile's reduction
-  // among workgroups through the caller's workspace: that is as fast at K = N = 4096 and faster on the FFN shapes
-  // (16 rows, N = 4096, K = 14336: 33 us against 52), and it feeds the matrix cores the reference's rounded weight.
+  // up to 16 rows of int8 codes (scale vectors through residue classes of the rows, one scale, none) or of int4
+  // codes in groups of 128 or more: one pass over the weight, whatever the compute type (16-bit compute types on
+  // the 16-bit matrix cores)
   bool few_rows_first = M <= 16 && (w_kind == CAIFX_W_INT8 || w_kind == CAIFX_W_INT4_GROUP);
-  if (few_rows_first && w_kind == CAIFX_W_INT4_GROUP && compute_dtype != CAIFX_F32 && !addend) {
-    const size_t shared = mfma_workspace_bytes(a, true);
-    if (shared > 0 && workspace && workspace_bytes >= shared) few_rows_first = false;
-  }
+#ifdef CAIFX_DEV
+  if (const char *e = getenv("CAIFX_DX_FEW")) few_rows_first = e[0] == '1' && M <= 16;
+#endif
   if (few_rows_first) {
     st = dxrows_backward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, dx, dx_dtype, M * K, stream);

@@ -2,9 +2,10 @@
 // bound on the weight stream like the decode forward, but with the reduction running down the weight's rows.
 //
 // v_mfma_f32_16x16x4_f32 holds one value per lane in both operands, so a weight row needs no transposition: a
-// lane (j = lane % 16, q = lane / 16) loads 8 consecutive codes of row n + q at k = k0 + 8j, and code b of that
+// lane (j = lane % 16, q = lane / 16) loads 8 consecutive codes of a row at k = k0 + 8j, and code b of that
 // load is the B operand of matrix instruction b, whose 16 columns are then k0 + 8*col + b.  The A operand is
-// dY[m = j][n + q].  Eight instructions consume one 8-byte load per lane; the sums stay in fp32, the codes are
+// dY[m = j][that row]; load i of a stage takes row 4q + i of the stage's 16 (which rows meet in one instruction
+// is free as long as both operands agree).  Eight instructions consume one 8-byte load per lane; the sums stay in fp32, the codes are
 // exact in fp32 and the weight's scale is applied to the finished column, so nothing is rounded to a 16-bit type
 // on the way (the reference rounds code*scale to the compute dtype first; results differ by that rounding, a
 // few 1e-3 of the largest output for bf16, 1e-7 for the fp32 compute type).
@@ -14,6 +15,9 @@
 // Packed int4 codes in groups of 128 or more take the same route with the scale on the other operand: a slab of
 // 128 columns lies inside one group, so the scale of (row, group) multiplies the row's gradient before it enters
 // the A operand.
+// With a 16-bit compute type the same loads feed v_mfma_f32_16x16x16 instead (four rows per instruction, a
+// sixteenth of the matrix time per code): the gradient is in that type already and int8 codes are exact in it, so
+// the sums are the same; int4 codes then meet their scale on the weight's side, rounded once to the compute type.
 //
 // A workgroup of 16 waves owns a slab of 128 columns (one cache line of every weight row it visits) and a range
 // of rows; the waves split the rows 16 at a time, add their 16 partial tiles through LDS in a fixed order and
@@ -51,15 +55,26 @@ struct DxArgs {
   int ranges;              // row ranges per class: blockIdx.y = cls * ranges + range
   int64_t rows_per_wg;     // rows of a class per workgroup
   float *partial;          // [gridDim.y][M][K] when the rows are split among workgroups, else null
+  int staged_pitch;        // GRAD_STAGED: elements per gradient row of the piece of dY kept in LDS
 };
 
 // XT: type of dY in memory; CT: compute type dY is rounded to first, as the layer's cast of its input does.
 // kInt4: packed int4 codes; a lane's 8 codes are one dword, and the scale of (row, group) multiplies the row's
 // gradient on its way into the A operand (the slab's 128 columns share the group).
-template <typename XT, typename CT, bool kInt4>
+// kGrad: how a lane gets its four gradient values of a stage (rows 4q .. 4q+3 of the stage's 16).  A wave's gradient
+// load touches 16 cache lines, one per gradient row, whatever its width, so four scalar loads per stage cost the
+// L1 four times what the weight loads do.
+//   GRAD_VECTOR  one load of four: the rows are neighbours in memory (no residue classes) and the vector is aligned
+//   GRAD_STAGED  residue classes put the rows V columns apart: the workgroup first copies its class's piece of dY
+//                into LDS (behind the first weight requests, which are in flight meanwhile) and reads four from there
+//   GRAD_SCALAR  four loads (whatever the other two do not take)
+enum { GRAD_SCALAR = 0, GRAD_VECTOR = 1, GRAD_STAGED = 2 };
+template <typename XT, typename CT, bool kInt4, int kGrad>
 __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
 {
-  extern __shared__ __attribute__((aligned(16))) float tiles[];      // [16 waves][8 codes][4][64], then [16][128] sums
+  constexpr bool kVecA = kGrad == GRAD_VECTOR;
+  // [16 waves][8 codes][4][64] partial tiles, then [16][128] sums; GRAD_STAGED: before those, the gradient piece
+  extern __shared__ __attribute__((aligned(16))) float tiles[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int j = lane & 15;
@@ -86,11 +101,33 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
   u32x2_t w[kDxStages][kDxIter];
   f16_t ws[kDxStages][kDxIter];          // int4: scale of the row in this slab's group
   XT av[kDxStages][kDxIter];             // dY as loaded
+  static_assert(kDxIter == 4, "a lane's gradient values of a stage are loaded as one vector of four");
+  struct alignas(4 * sizeof(XT)) XT4 {
+    XT v[4];
+  };
   uint32_t keep[kDxStages][kDxIter];     // all ones where the row and the gradient row exist, else 0
+  // GRAD_STAGED: staged[m][i - n_lo] for the rows i of this workgroup's range, zero past the range's end; the row
+  // pitch is 16 bytes past a multiple of 256, so the 16 gradient rows of one pass of a read use different banks
+  const int staged_pitch = a.staged_pitch;          // elements
+  XT *staged = reinterpret_cast<XT *>(tiles);
+  auto issue_a = [&](int st, int64_t base) {
+    if constexpr (kVecA) {        // V == 1: rows base + 4q .. + 3 are four consecutive gradient columns
+      const int64_t n4 = base + 4 * q;
+      const XT4 g4 = *reinterpret_cast<const XT4 *>(dy + (n4 + 4 <= a.N ? n4 : a.N - 4));       // past the end: masked below
+#pragma unroll
+      for (int it = 0; it < kDxIter; ++it) av[st][it] = g4.v[it];
+    } else if constexpr (kGrad == GRAD_STAGED) {
+      int64_t i4 = base - n_lo + 4 * q;
+      if (i4 > staged_pitch - 4) i4 = staged_pitch - 4;       // passes past the range read the zeros at its end
+      const XT4 g4 = *reinterpret_cast<const XT4 *>(staged + j * staged_pitch + i4);
+#pragma unroll
+      for (int it = 0; it < kDxIter; ++it) av[st][it] = g4.v[it];
+    }
+  };
   auto issue = [&](int st, int64_t base) {
 #pragma unroll
     for (int it = 0; it < kDxIter; ++it) {
-      const int64_t n = base + 4 * it + q;
+      const int64_t n = base + 4 * q + it;
       const int64_t nn = cls + a.V * (n < n_hi ? n : n_hi - 1);          // rows past the range: a valid address, a zero gradient
       if constexpr (kInt4) {
         w[st][it][0] = *reinterpret_cast<const uint32_t *>(wcol + nn * row_bytes);
@@ -98,13 +135,61 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
       } else {
         w[st][it] = *reinterpret_cast<const u32x2_t *>(wcol + nn * row_bytes);
       }
-      av[st][it] = dy[nn];
+      if constexpr (kGrad == GRAD_SCALAR) av[st][it] = dy[nn];
       // (a mask on the bits, not a conditional expression: the compiler turns that into a load under a branch
       // with a full wait behind it)
       keep[st][it] = static_cast<uint32_t>(-static_cast<int>((n < n_hi) & row_live));
     }
   };
+  // 16-bit compute types: one v_mfma_f32_16x16x16 per code position takes the stage's four rows at once.  Its lanes
+  // hold four consecutive reduction elements; which weight rows those are is free as long as both operands agree,
+  // so element e of lane (j, q) is row 4q + e of the stage: the loads above as they are.  The gradient is in the
+  // compute type already and an int8 code is exact in it, so the sums are those of the fp32 form; an int4 code meets
+  // its scale on this side, code * scale rounded once to the compute type: the reference's dequantised weight.
+  auto multiply16 = [&](int st) {
+   if constexpr (sizeof(CT) == 2) {
+    typedef short short4_t __attribute__((ext_vector_type(4)));
+    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+    float g[kDxIter];
+#pragma unroll
+    for (int it = 0; it < kDxIter; ++it)
+      g[it] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, to_f32<XT>(av[st][it])) & keep[st][it]);
+    u32x2_t av2;
+    av2[0] = pack2<CT>(g[0], g[1]);
+    av2[1] = pack2<CT>(g[2], g[3]);
+    float c[kDxIter][8];
+#pragma unroll
+    for (int it = 0; it < kDxIter; ++it) {
+      if constexpr (kInt4) {
+        dequant_int4x8(w[st][it][0], to_f32(ws[st][it]), c[it]);
+      } else {
+        float lo[4], hi[4];
+        int8x4_to_f32(w[st][it][0], lo);
+        int8x4_to_f32(w[st][it][1], hi);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          c[it][b] = lo[b];
+          c[it][4 + b] = hi[b];
+        }
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      u32x2_t bv;
+      bv[0] = pack2<CT>(c[0][b], c[1][b]);
+      bv[1] = pack2<CT>(c[2][b], c[3][b]);
+      if constexpr (dtype_code<CT>::value == CAIFX_BF16)
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, av2), __builtin_bit_cast(short4_t, bv), acc[b], 0, 0, 0);
+      else
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, av2), __builtin_bit_cast(half4_t, bv), acc[b], 0, 0, 0);
+    }
+   }
+  };
   auto multiply = [&](int st) {
+    if constexpr (sizeof(CT) == 2) {
+      multiply16(st);
+      return;
+    }
 #pragma unroll
     for (int it = 0; it < kDxIter; ++it) {
       float g = round_through<CT>(to_f32<XT>(av[st][it]));
@@ -123,16 +208,42 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
   // to save registers, with a full wait in front of every multiplication)
 #pragma unroll
   for (int st = 0; st < kDxStages - 1; ++st) issue(st, base + st * kDxPassRows);
+  if constexpr (kGrad == GRAD_STAGED) {
+    // the piece of dY this workgroup's rows meet: 16 gradient rows (zero from M on) x the range's rows of the class
+    // (eight loads at a time per thread, all issued before the first is stored: one at a time the copy would take
+    // a memory round trip per element)
+    const XT *src = static_cast<const XT *>(a.dy) + cls + a.V * n_lo;
+    const int64_t last = (n_hi - n_lo - 1) * a.V;            // offset of the range's last row
+    for (int i0 = 0; i0 < staged_pitch; i0 += kDxThreads) {
+      const int i = i0 + static_cast<int>(threadIdx.x);
+      const int64_t off = static_cast<int64_t>(i) * a.V;
+      const XT *col = src + (off < last ? off : last);
+#pragma unroll
+      for (int m0 = 0; m0 < 16; m0 += 8) {
+        XT v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = col[static_cast<int64_t>(m0 + u < a.M ? m0 + u : a.M - 1) * a.N];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (i < staged_pitch) staged[(m0 + u) * staged_pitch + i] = (m0 + u < a.M && n_lo + i < n_hi) ? v[u] : from_f32<XT>(0.0f);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int st = 0; st < kDxStages - 1; ++st) issue_a(st, base + st * kDxPassRows);
   for (; base < n_hi; base += kDxStages * kDxPassRows) {       // the same trip count for every lane of a wave
 #pragma unroll
     for (int st = 0; st < kDxStages; ++st) {
       issue((st + kDxStages - 1) % kDxStages, base + (st + kDxStages - 1) * kDxPassRows);
+      issue_a((st + kDxStages - 1) % kDxStages, base + (st + kDxStages - 1) * kDxPassRows);
       __builtin_amdgcn_sched_barrier(0);
       multiply(st);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
 
+  if constexpr (kGrad == GRAD_STAGED) __syncthreads();      // the partial tiles go where other waves may still read gradients
   // acc[b][v] = this wave's share of dX[4*(lane/16) + v][k0 + 8*(lane%16) + b]
 #pragma unroll
   for (int b = 0; b < 8; ++b)
@@ -187,13 +298,37 @@ int compute_units()
   return 256;
 }
 
+template <typename XT, typename CT, bool kInt4>
+int launch_vec(const DxArgs &a, dim3 grid, size_t lds, hipStream_t s)
+{
+  // one vector load per stage for the gradient when its four values are neighbours and the vector is aligned;
+  // with residue classes the workgroup's piece of dY goes through LDS when it fits where the partial tiles go later
+  const bool vec = a.V == 1 && a.N % 4 == 0 && a.N >= 4 && aligned_to(a.dy, 4 * sizeof(XT));
+  if (vec) {
+    hipLaunchKernelGGL((dxrows_kernel<XT, CT, kInt4, GRAD_VECTOR>), grid, dim3(kDxThreads), lds, s, a);
+    return launch_status();
+  }
+  if (a.V > 1 && a.M > 1) {
+    // pitch: the range's rows, rounded up to 16 bytes past a multiple of 256
+    const int64_t per256 = 256 / static_cast<int64_t>(sizeof(XT));
+    const int64_t pitch = (a.rows_per_wg + per256 - 1) / per256 * per256 + 16 / static_cast<int64_t>(sizeof(XT));
+    if (16 * pitch * sizeof(XT) <= lds) {
+      DxArgs b = a;
+      b.staged_pitch = static_cast<int>(pitch);
+      hipLaunchKernelGGL((dxrows_kernel<XT, CT, kInt4, GRAD_STAGED>), grid, dim3(kDxThreads), lds, s, b);
+      return launch_status();
+    }
+  }
+  hipLaunchKernelGGL((dxrows_kernel<XT, CT, kInt4, GRAD_SCALAR>), grid, dim3(kDxThreads), lds, s, a);
+  return launch_status();
+}
+
 template <typename CT, bool kInt4>
 int launch_xt(const DxArgs &a, int x_dtype, dim3 grid, size_t lds, hipStream_t s)
 {
-  if (x_dtype == CAIFX_F32) hipLaunchKernelGGL((dxrows_kernel<float, CT, kInt4>), grid, dim3(kDxThreads), lds, s, a);
-  else if (x_dtype == CAIFX_BF16) hipLaunchKernelGGL((dxrows_kernel<bf16_t, CT, kInt4>), grid, dim3(kDxThreads), lds, s, a);
-  else hipLaunchKernelGGL((dxrows_kernel<f16_t, CT, kInt4>), grid, dim3(kDxThreads), lds, s, a);
-  return launch_status();
+  if (x_dtype == CAIFX_F32) return launch_vec<float, CT, kInt4>(a, grid, lds, s);
+  if (x_dtype == CAIFX_BF16) return launch_vec<bf16_t, CT, kInt4>(a, grid, lds, s);
+  return launch_vec<f16_t, CT, kInt4>(a, grid, lds, s);
 }
 
 template <typename CT>
@@ -241,10 +376,23 @@ DxPlan plan(const GemmArgs &g)
   const int64_t slabs = g.K / kDxSlab;
   static const int cus = compute_units();
   const int64_t rows_class = (g.N + p.V - 1) / p.V;                 // of the largest class
-  int64_t ranges = (cus + slabs * p.V - 1) / (slabs * p.V);
+  // Row ranges per class: one workgroup fills a compute unit (its partial tiles take 128 KB of LDS), so the launch
+  // runs in rounds of `cus` workgroups, each round as long as a range plus what a workgroup spends before and after
+  // its rows (about 470 rows' worth of streaming).  The fewest rounds of the shortest ranges win: 16 rows, N = 4096,
+  // K = 14336, int8 in two classes (224 workgroups per range): one range 22.7 us, two 27.3, three 33.6; int4 (112):
+  // one 32.8, two 21.9, three 31.0.
   const int64_t most = (rows_class + kDxPassRows - 1) / kDxPassRows;      // every workgroup gets at least one full pass
-  if (ranges > most) ranges = most;
-  if (ranges < 1) ranges = 1;
+  const int64_t items = slabs * p.V;
+  int64_t ranges = 1;
+  int64_t best = -1;
+  for (int64_t r = 1; r <= most && r <= 64; ++r) {
+    const int64_t rounds = (items * r + cus - 1) / cus;
+    const int64_t cost = rounds * (rows_class / r + 470);
+    if (best < 0 || cost < best) {
+      best = cost;
+      ranges = r;
+    }
+  }
   int64_t rows = (rows_class + ranges - 1) / ranges;
   rows = (rows + kDxWaveRows - 1) / kDxWaveRows * kDxWaveRows;
   p.rows_per_wg = rows;

@@ -148,11 +148,11 @@ CAIFX_API int caifx_qlinear_forward(int64_t M, int64_t N, int64_t K,
  *   dX[M,K] = cast<compute>(dY)[M,N] * cast<compute>(dequant(W))[N,K], fp32 accumulate.
  * With up to 16 rows and int8 codes (any scale vector that leaves at most 64 residue classes of rows with
  * equal scales along k, each of 256 rows or more; one scale; none) or int4 codes in groups of 128 or more, the
- * weight is streamed once through
- * the fp32 matrix core and its scale is applied outside the products: like the forward's memory-bound kernels
- * this skips the rounding of
- * code * scale to a 16-bit compute type (about 2e-3 of max|dX| for bf16; for the fp32 compute type the
- * difference is fp32 rounding, 1e-7). */
+ * weight is streamed once through the matrix cores (the 16-bit ones for a 16-bit compute type, the fp32 one
+ * for fp32).  For int8 codes the scale is applied outside the products: like the forward's memory-bound kernels
+ * this skips the rounding of code * scale to a 16-bit compute type (about 2e-3 of max|dX| for bf16; for the
+ * fp32 compute type the difference is fp32 rounding, 1e-7).  int4 codes with a 16-bit compute type meet their
+ * scale before the product, rounded once to the compute type: the reference's operand. */
 CAIFX_API int caifx_qlinear_backward_input(int64_t M, int64_t N, int64_t K,
                                  const void *dy, int dy_dtype, int compute_dtype,
                                  const void *wq, int w_kind, const void *scales, int64_t scale_period,
@@ -195,9 +195,8 @@ CAIFX_API int caifx_qlinear_backward_input_add(int64_t M, int64_t N, int64_t K,
  * workspace also selects between the two accuracy classes of caifx_qlinear_forward's comment: the input gradient
  * with up to 16 rows and the forward with up to 16 rows and K > 4096 run, without it, on kernels that round
  * code * scale to the 16-bit compute type as the reference does, and with it on the few-row kernels that multiply
- * unrounded codes (about 2e-3 of max|out| apart; both within the 1e-2 bound).  Packed int4 with a 16-bit compute
- * type is the other way round for the input gradient: with the workspace it takes the tiled kernel (rounded
- * weight), without it the few-row kernel when that needs no workspace. */
+ * unrounded codes (about 2e-3 of max|out| apart; both within the 1e-2 bound; the few-row input gradient of packed
+ * int4 with a 16-bit compute type multiplies the rounded weight either way). */
 CAIFX_API size_t caifx_qlinear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtype, int compute_dtype,
                                      int w_kind, int backward);
 

@@ -337,6 +337,16 @@ def test_input_gradient_few_rows_dtype_mixes(orc, cd, xd, yd):
             assert err <= TIGHT_POST
 
 
+@pytest.mark.parametrize("cd", [1, 2])
+def test_input_gradient_few_rows_int4_multiplies_the_rounded_weight(orc, cd):
+    # 16-bit compute types run the few-row kernel on the 16-bit matrix cores; int4 codes meet their scale before the
+    # product, rounded once to the compute type, so the operands are the oracle's and only the order of the fp32 sums
+    # differs.  N = 1000 leaves a last stage with 8 of 16 rows; M = 1 and a gradient given in fp32.
+    rng = np.random.default_rng(90 + cd)
+    for M, N, K, xd in ((16, 4096, 4096, cd), (7, 640, 1280, cd), (3, 1000, 1024, 0), (1, 2048, 256, cd)):
+        assert _check_dx(orc, rng, M, N, K, "int4", cd, xd) <= TIGHT_16, (M, N, K)
+
+
 def test_input_gradient_few_rows_other_paths(orc):
     # per-channel scales whose index depends on the weight row in too many ways (205 residue classes), int4 groups
     # below 128, more than 16 rows and a call without a workspace go to the tiled kernels; all must agree with the oracle
