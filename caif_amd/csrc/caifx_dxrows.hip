@@ -1,23 +1,25 @@
 // Input gradient for a handful of rows (M <= 16): dX[M,K] = dY[M,N] * W[N,K] with W stored as int8 codes, memory
 // bound on the weight stream like the decode forward, but with the reduction running down the weight's rows.
 //
-// v_mfma_f32_16x16x4_f32 holds one value per lane in both operands, so a weight row needs no transposition: a
-// lane (j = lane % 16, q = lane / 16) loads 8 consecutive codes of a row at k = k0 + 8j, and code b of that
-// load is the B operand of matrix instruction b, whose 16 columns are then k0 + 8*col + b.  The A operand is
-// dY[m = j][that row]; load i of a stage takes row 4q + i of the stage's 16 (which rows meet in one instruction
-// is free as long as both operands agree).  Eight instructions consume one 8-byte load per lane; the sums stay in fp32, the codes are
-// exact in fp32 and the weight's scale is applied to the finished column, so nothing is rounded to a 16-bit type
-// on the way (the reference rounds code*scale to the compute dtype first; results differ by that rounding, a
-// few 1e-3 of the largest output for bf16, 1e-7 for the fp32 compute type).
-// That needs the scale of W[n][k] not to depend on n among the rows a workgroup visits: scale index
+// The 16-bit and integer matrix instructions hold several consecutive reduction elements of one column per lane,
+// here several weight rows of one column, while a weight row is stored along k.  v_mfma_f32_16x16x16 (bf16 / fp16)
+// holds four: lane (j = lane % 16, q = lane / 16) loads 8 consecutive codes of four rows at k = k0 + 8j (four
+// 8-byte loads, row 4q + i of the stage's 16 for load i; which rows meet in one instruction is free as long as
+// both operands agree), and code position b of the four loads is the B operand of matrix instruction b, whose 16
+// columns are then k0 + 8*col + b: no transposition, the byte (or nibble) is picked when the code is converted.
+// The A operand is dY[m = j][those four rows].  Eight instructions consume a stage of four loads per lane.
+//   * 16-bit compute type: dY is in that type (or rounded to it first, as the layer's cast of its input does), int8
+//     codes are exact in it and the weight's scale is applied to the finished column, so the weight is never rounded
+//     to the compute type (the reference rounds code*scale first; results differ by that rounding, a few 1e-3 of the
+//     largest output for bf16).  int4 codes meet their scale before the product, code * scale rounded once to the
+//     compute type: the reference's operand.
+//   * fp32 compute type: dY (times the int4 scale) is cut into three bf16 pieces that add up to it, the codes are
+//     exact in bf16, and three instructions per code position form the fp32 products (1e-7 of the largest output).
+// The scale of an int8 column must not depend on the weight row among the rows a workgroup visits: scale index
 // (n*K + k) mod period with K a multiple of the period (the per-output-channel scales of a square weight), one
 // scale, none, or any period with the rows split into residue classes (see DxArgs::V).
-// Packed int4 codes in groups of 128 or more take the same route with the scale on the other operand: a slab of
-// 128 columns lies inside one group, so the scale of (row, group) multiplies the row's gradient before it enters
-// the A operand.
-// With a 16-bit compute type the same loads feed v_mfma_f32_16x16x16 instead (four rows per instruction, a
-// sixteenth of the matrix time per code): the gradient is in that type already and int8 codes are exact in it, so
-// the sums are the same; int4 codes then meet their scale on the weight's side, rounded once to the compute type.
+// Packed int4 codes come in groups of 128 or more: a slab of 128 columns lies inside one group, so a row has one
+// scale per slab (fp32 compute: it multiplies the row's gradient on its way into the A operand).
 //
 // A workgroup of 16 waves owns a slab of 128 columns (one cache line of every weight row it visits) and a range
 // of rows; the waves split the rows 16 at a time, add their 16 partial tiles through LDS in a fixed order and
@@ -30,9 +32,9 @@ namespace {
 constexpr int kDxWaves = 16;
 constexpr int kDxThreads = kDxWaves * 64;
 constexpr int kDxSlab = 128;                 // columns of dX per workgroup
-// 8-byte weight loads per stage of a wave's ring (4 rows each) and stages.  Measured at N = K = 4096 / N = 14336,
-// 16 rows: 4 x 2: 15.6 / 33.4 us; 2 x 4: 16.1 / 32.6; 4 x 3: 19.8 / 36.5; 4 x 4: 24.4 / 35.6; 8 x 2: 23.4 / 35.5
-// (a deeper ring only adds passes past the last row, which still cost their multiplications).
+// 8-byte weight loads per stage of a wave's ring (the four rows of one matrix instruction) and stages.  Three
+// stages measured slower than two at every shape (16 rows of int8: 12.1 -> 13.8 us at N = K = 4096, 22.2 -> 22.8 at
+// N = 4096 / K = 14336, 24.1 -> 25.0 at N = 14336 / K = 4096; int4 21.8 -> 23.3).
 constexpr int kDxIter = 4;
 constexpr int kDxStages = 2;
 constexpr int kDxWaveRows = 4 * kDxIter;     // rows a wave takes per pass
@@ -185,22 +187,55 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
     }
    }
   };
+  // fp32 compute type: the gradient (times the int4 scale) is cut into three bf16 pieces, g = h + m + l to the last
+  // bit of its mantissa or better (each piece is the rounded remainder of the one before, and the remainders are
+  // exact), the codes are exact in bf16, so three v_mfma_f32_16x16x16 per code position form the same fp32 products
+  // as 32 v_mfma_f32_16x16x4_f32 would, in a third of the matrix time.
+  auto multiply_split = [&](int st) {
+    typedef short short4_t __attribute__((ext_vector_type(4)));
+    float h[kDxIter], m[kDxIter], l[kDxIter];
+#pragma unroll
+    for (int it = 0; it < kDxIter; ++it) {
+      float g = to_f32<XT>(av[st][it]);
+      if constexpr (kInt4) g *= to_f32(ws[st][it]);
+      g = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, g) & keep[st][it]);
+      h[it] = round_through<bf16_t>(g);
+      const float r1 = g - h[it];
+      m[it] = round_through<bf16_t>(r1);
+      l[it] = r1 - m[it];               // rounded to bf16 by the pack below
+    }
+    u32x2_t ah, am, al;
+    ah[0] = pack2<bf16_t>(h[0], h[1]);
+    ah[1] = pack2<bf16_t>(h[2], h[3]);
+    am[0] = pack2<bf16_t>(m[0], m[1]);
+    am[1] = pack2<bf16_t>(m[2], m[3]);
+    al[0] = pack2<bf16_t>(l[0], l[1]);
+    al[1] = pack2<bf16_t>(l[2], l[3]);
+    float c[kDxIter][8];
+#pragma unroll
+    for (int it = 0; it < kDxIter; ++it)
+#pragma unroll
+      for (int b = 0; b < 8; ++b)
+        c[it][b] = static_cast<float>(kInt4 ? static_cast<int>(w[st][it][0] << (28 - 4 * b)) >> 28
+                                            : static_cast<int>(w[st][it][b >> 2] << (24 - 8 * (b & 3))) >> 24);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      u32x2_t bv;
+      bv[0] = pack2<bf16_t>(c[0][b], c[1][b]);
+      bv[1] = pack2<bf16_t>(c[2][b], c[3][b]);
+      const short4_t bb = __builtin_bit_cast(short4_t, bv);
+      // smallest piece first
+      acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, al), bb, acc[b], 0, 0, 0);
+      acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, am), bb, acc[b], 0, 0, 0);
+      acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, ah), bb, acc[b], 0, 0, 0);
+    }
+  };
   auto multiply = [&](int st) {
     if constexpr (sizeof(CT) == 2) {
       multiply16(st);
       return;
-    }
-#pragma unroll
-    for (int it = 0; it < kDxIter; ++it) {
-      float g = round_through<CT>(to_f32<XT>(av[st][it]));
-      if constexpr (kInt4) g *= to_f32(ws[st][it]);
-      g = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, g) & keep[st][it]);
-#pragma unroll
-      for (int b = 0; b < 8; ++b) {
-        const int code = kInt4 ? static_cast<int>(w[st][it][0] << (28 - 4 * b)) >> 28
-                               : static_cast<int>(w[st][it][b >> 2] << (24 - 8 * (b & 3))) >> 24;
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(g, static_cast<float>(code), acc[b], 0, 0, 0);
-      }
+    } else {
+      multiply_split(st);
     }
   };
   int64_t base = n_lo + static_cast<int64_t>(wave) * kDxWaveRows;
@@ -312,10 +347,11 @@ int launch_vec(const DxArgs &a, dim3 grid, size_t lds, hipStream_t s)
     // pitch: the range's rows, rounded up to 16 bytes past a multiple of 256
     const int64_t per256 = 256 / static_cast<int64_t>(sizeof(XT));
     const int64_t pitch = (a.rows_per_wg + per256 - 1) / per256 * per256 + 16 / static_cast<int64_t>(sizeof(XT));
-    if (16 * pitch * sizeof(XT) <= lds) {
+    const size_t piece = 16 * static_cast<size_t>(pitch) * sizeof(XT);
+    if (piece <= 160 * 1024) {
       DxArgs b = a;
       b.staged_pitch = static_cast<int>(pitch);
-      hipLaunchKernelGGL((dxrows_kernel<XT, CT, kInt4, GRAD_STAGED>), grid, dim3(kDxThreads), lds, s, b);
+      hipLaunchKernelGGL((dxrows_kernel<XT, CT, kInt4, GRAD_STAGED>), grid, dim3(kDxThreads), piece > lds ? piece : lds, s, b);
       return launch_status();
     }
   }
