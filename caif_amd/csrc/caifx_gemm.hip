@@ -31,6 +31,41 @@ __global__ void splitk_reduce_kernel(const float *__restrict__ partial, int part
   y[i] = from_f32<T>(v);
 }
 
+// The same for four neighbouring elements per thread (n a multiple of 4, 16-byte aligned partial sums): the parts
+// are requested four at a time before the first is added, in the same order of additions.
+template <typename T>
+__global__ void splitk_reduce_x4_kernel(const float *__restrict__ partial, int parts, int64_t n, T *__restrict__ y,
+                                        const T *__restrict__ addend)
+{
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+  if (i >= n) return;
+  const floatx4_t *src = reinterpret_cast<const floatx4_t *>(partial + i);
+  const int64_t stride = n >> 2;
+  floatx4_t v = src[0];
+  int p = 1;
+  for (; p + 4 <= parts; p += 4) {
+    const floatx4_t a = src[p * stride], b = src[(p + 1) * stride], c = src[(p + 2) * stride], d = src[(p + 3) * stride];
+    v += a;
+    v += b;
+    v += c;
+    v += d;
+  }
+  for (; p < parts; ++p) v += src[p * stride];
+  struct alignas(4 * sizeof(T)) T4 {
+    T e[4];
+  };
+  T4 out;
+  if (addend) {
+    const T4 add = *reinterpret_cast<const T4 *>(addend + i);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out.e[e] = from_f32<T>(round_through<T>(v[e]) + to_f32<T>(add.e[e]));
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out.e[e] = from_f32<T>(v[e]);
+  }
+  *reinterpret_cast<T4 *>(y + i) = out;
+}
+
 // With no more tiles than compute units the launch lasts one tile's whole reduction (43-70 us at K = 4096) however
 // few rows there are.  Then up to 8 workgroups share a tile's reduction, each at least 8 steps of it, and write
 // fp32 partial tiles to the caller's workspace; a second launch adds them in a fixed order.
@@ -171,6 +206,20 @@ int run(const GemmArgs &a, bool backward, hipStream_t s)
 
 int splitk_reduce(const float *partial, int parts, int64_t n, void *y, int y_dtype, const void *addend, hipStream_t s)
 {
+  const size_t quad = 4 * (y_dtype == CAIFX_F32 ? 4 : 2);
+  if (n % 4 == 0 && aligned_to(partial, 16) && aligned_to(y, quad) && (!addend || aligned_to(addend, quad))) {
+    const dim3 grid4(static_cast<unsigned>((n / 4 + 255) / 256));
+    if (y_dtype == CAIFX_F32)
+      hipLaunchKernelGGL(splitk_reduce_x4_kernel<float>, grid4, dim3(256), 0, s, partial, parts, n, static_cast<float *>(y),
+                         static_cast<const float *>(addend));
+    else if (y_dtype == CAIFX_BF16)
+      hipLaunchKernelGGL(splitk_reduce_x4_kernel<bf16_t>, grid4, dim3(256), 0, s, partial, parts, n, static_cast<bf16_t *>(y),
+                         static_cast<const bf16_t *>(addend));
+    else
+      hipLaunchKernelGGL(splitk_reduce_x4_kernel<f16_t>, grid4, dim3(256), 0, s, partial, parts, n, static_cast<f16_t *>(y),
+                         static_cast<const f16_t *>(addend));
+    return launch_status();
+  }
   const dim3 grid(static_cast<unsigned>((n + 255) / 256));
   if (y_dtype == CAIFX_F32)
     hipLaunchKernelGGL(splitk_reduce_kernel<float>, grid, dim3(256), 0, s, partial, parts, n, static_cast<float *>(y),
