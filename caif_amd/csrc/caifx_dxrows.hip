@@ -35,7 +35,10 @@ constexpr int kDxSlab = 128;                 // columns of dX per workgroup
 // 8-byte weight loads per stage of a wave's ring (the four rows of one matrix instruction) and stages.  Three
 // stages measured slower than two at every shape (16 rows of int8: 12.1 -> 13.8 us at N = K = 4096, 22.2 -> 22.8 at
 // N = 4096 / K = 14336, 24.1 -> 25.0 at N = 14336 / K = 4096; int4 21.8 -> 23.3).
-constexpr int kDxIter = 4;
+// matrix instructions' worth of rows (four each) a lane loads per stage; two measured slower or equal at every shape
+// (16 rows of int8, N = K = 4096: 11.2 -> 14.8 us; int4, N = 4096 / K = 14336: 21.7 -> 25.0)
+constexpr int kDxGroups = 1;
+constexpr int kDxIter = 4 * kDxGroups;
 constexpr int kDxStages = 2;
 constexpr int kDxWaveRows = 4 * kDxIter;     // rows a wave takes per pass
 constexpr int kDxPassRows = kDxWaves * kDxWaveRows;
@@ -103,9 +106,8 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
   u32x2_t w[kDxStages][kDxIter];
   f16_t ws[kDxStages][kDxIter];          // int4: scale of the row in this slab's group
   XT av[kDxStages][kDxIter];             // dY as loaded
-  static_assert(kDxIter == 4, "a lane's gradient values of a stage are loaded as one vector of four");
-  struct alignas(4 * sizeof(XT)) XT4 {
-    XT v[4];
+  struct alignas(kDxIter * sizeof(XT) > 16 ? 16 : kDxIter * sizeof(XT)) XT4 {      // a lane's gradient values of a stage
+    XT v[kDxIter];
   };
   uint32_t keep[kDxStages][kDxIter];     // all ones where the row and the gradient row exist, else 0
   // GRAD_STAGED: staged[m][i - n_lo] for the rows i of this workgroup's range, zero past the range's end; the row
@@ -114,13 +116,13 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
   XT *staged = reinterpret_cast<XT *>(tiles);
   auto issue_a = [&](int st, int64_t base) {
     if constexpr (kVecA) {        // V == 1: rows base + 4q .. + 3 are four consecutive gradient columns
-      const int64_t n4 = base + 4 * q;
-      const XT4 g4 = *reinterpret_cast<const XT4 *>(dy + (n4 + 4 <= a.N ? n4 : a.N - 4));       // past the end: masked below
+      const int64_t n4 = base + kDxIter * q;
+      const XT4 g4 = *reinterpret_cast<const XT4 *>(dy + (n4 + kDxIter <= a.N ? n4 : a.N - kDxIter));       // past the end: masked below
 #pragma unroll
       for (int it = 0; it < kDxIter; ++it) av[st][it] = g4.v[it];
     } else if constexpr (kGrad == GRAD_STAGED) {
-      int64_t i4 = base - n_lo + 4 * q;
-      if (i4 > staged_pitch - 4) i4 = staged_pitch - 4;       // passes past the range read the zeros at its end
+      int64_t i4 = base - n_lo + kDxIter * q;
+      if (i4 > staged_pitch - kDxIter) i4 = staged_pitch - kDxIter;       // passes past the range read the zeros at its end
       const XT4 g4 = *reinterpret_cast<const XT4 *>(staged + j * staged_pitch + i4);
 #pragma unroll
       for (int it = 0; it < kDxIter; ++it) av[st][it] = g4.v[it];
@@ -129,7 +131,7 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
   auto issue = [&](int st, int64_t base) {
 #pragma unroll
     for (int it = 0; it < kDxIter; ++it) {
-      const int64_t n = base + 4 * q + it;
+      const int64_t n = base + kDxIter * q + it;
       const int64_t nn = cls + a.V * (n < n_hi ? n : n_hi - 1);          // rows past the range: a valid address, a zero gradient
       if constexpr (kInt4) {
         w[st][it][0] = *reinterpret_cast<const uint32_t *>(wcol + nn * row_bytes);
@@ -152,38 +154,42 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
    if constexpr (sizeof(CT) == 2) {
     typedef short short4_t __attribute__((ext_vector_type(4)));
     typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-    float g[kDxIter];
 #pragma unroll
-    for (int it = 0; it < kDxIter; ++it)
-      g[it] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, to_f32<XT>(av[st][it])) & keep[st][it]);
-    u32x2_t av2;
-    av2[0] = pack2<CT>(g[0], g[1]);
-    av2[1] = pack2<CT>(g[2], g[3]);
-    float c[kDxIter][8];
+    for (int grp = 0; grp < kDxGroups; ++grp) {
+      float g[4];
 #pragma unroll
-    for (int it = 0; it < kDxIter; ++it) {
-      if constexpr (kInt4) {
-        dequant_int4x8(w[st][it][0], to_f32(ws[st][it]), c[it]);
-      } else {
-        float lo[4], hi[4];
-        int8x4_to_f32(w[st][it][0], lo);
-        int8x4_to_f32(w[st][it][1], hi);
+      for (int e = 0; e < 4; ++e)
+        g[e] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, to_f32<XT>(av[st][4 * grp + e])) & keep[st][4 * grp + e]);
+      u32x2_t av2;
+      av2[0] = pack2<CT>(g[0], g[1]);
+      av2[1] = pack2<CT>(g[2], g[3]);
+      float c[4][8];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          c[it][b] = lo[b];
-          c[it][4 + b] = hi[b];
+      for (int e = 0; e < 4; ++e) {
+        const int it = 4 * grp + e;
+        if constexpr (kInt4) {
+          dequant_int4x8(w[st][it][0], to_f32(ws[st][it]), c[e]);
+        } else {
+          float lo[4], hi[4];
+          int8x4_to_f32(w[st][it][0], lo);
+          int8x4_to_f32(w[st][it][1], hi);
+#pragma unroll
+          for (int b = 0; b < 4; ++b) {
+            c[e][b] = lo[b];
+            c[e][4 + b] = hi[b];
+          }
         }
       }
-    }
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
-      u32x2_t bv;
-      bv[0] = pack2<CT>(c[0][b], c[1][b]);
-      bv[1] = pack2<CT>(c[2][b], c[3][b]);
-      if constexpr (dtype_code<CT>::value == CAIFX_BF16)
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, av2), __builtin_bit_cast(short4_t, bv), acc[b], 0, 0, 0);
-      else
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, av2), __builtin_bit_cast(half4_t, bv), acc[b], 0, 0, 0);
+      for (int b = 0; b < 8; ++b) {
+        u32x2_t bv;
+        bv[0] = pack2<CT>(c[0][b], c[1][b]);
+        bv[1] = pack2<CT>(c[2][b], c[3][b]);
+        if constexpr (dtype_code<CT>::value == CAIFX_BF16)
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, av2), __builtin_bit_cast(short4_t, bv), acc[b], 0, 0, 0);
+        else
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, av2), __builtin_bit_cast(half4_t, bv), acc[b], 0, 0, 0);
+      }
     }
    }
   };
@@ -193,41 +199,45 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
   // as 32 v_mfma_f32_16x16x4_f32 would, in a third of the matrix time.
   auto multiply_split = [&](int st) {
     typedef short short4_t __attribute__((ext_vector_type(4)));
-    float h[kDxIter], m[kDxIter], l[kDxIter];
 #pragma unroll
-    for (int it = 0; it < kDxIter; ++it) {
-      float g = to_f32<XT>(av[st][it]);
-      if constexpr (kInt4) g *= to_f32(ws[st][it]);
-      g = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, g) & keep[st][it]);
-      h[it] = round_through<bf16_t>(g);
-      const float r1 = g - h[it];
-      m[it] = round_through<bf16_t>(r1);
-      l[it] = r1 - m[it];               // rounded to bf16 by the pack below
-    }
-    u32x2_t ah, am, al;
-    ah[0] = pack2<bf16_t>(h[0], h[1]);
-    ah[1] = pack2<bf16_t>(h[2], h[3]);
-    am[0] = pack2<bf16_t>(m[0], m[1]);
-    am[1] = pack2<bf16_t>(m[2], m[3]);
-    al[0] = pack2<bf16_t>(l[0], l[1]);
-    al[1] = pack2<bf16_t>(l[2], l[3]);
-    float c[kDxIter][8];
+    for (int grp = 0; grp < kDxGroups; ++grp) {
+      float h[4], m[4], l[4];
 #pragma unroll
-    for (int it = 0; it < kDxIter; ++it)
+      for (int e = 0; e < 4; ++e) {
+        const int it = 4 * grp + e;
+        float g = to_f32<XT>(av[st][it]);
+        if constexpr (kInt4) g *= to_f32(ws[st][it]);
+        g = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, g) & keep[st][it]);
+        h[e] = round_through<bf16_t>(g);
+        const float r1 = g - h[e];
+        m[e] = round_through<bf16_t>(r1);
+        l[e] = r1 - m[e];               // rounded to bf16 by the pack below
+      }
+      u32x2_t ah, am, al;
+      ah[0] = pack2<bf16_t>(h[0], h[1]);
+      ah[1] = pack2<bf16_t>(h[2], h[3]);
+      am[0] = pack2<bf16_t>(m[0], m[1]);
+      am[1] = pack2<bf16_t>(m[2], m[3]);
+      al[0] = pack2<bf16_t>(l[0], l[1]);
+      al[1] = pack2<bf16_t>(l[2], l[3]);
+      float c[4][8];
 #pragma unroll
-      for (int b = 0; b < 8; ++b)
-        c[it][b] = static_cast<float>(kInt4 ? static_cast<int>(w[st][it][0] << (28 - 4 * b)) >> 28
-                                            : static_cast<int>(w[st][it][b >> 2] << (24 - 8 * (b & 3))) >> 24);
+      for (int e = 0; e < 4; ++e)
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
-      u32x2_t bv;
-      bv[0] = pack2<bf16_t>(c[0][b], c[1][b]);
-      bv[1] = pack2<bf16_t>(c[2][b], c[3][b]);
-      const short4_t bb = __builtin_bit_cast(short4_t, bv);
-      // smallest piece first
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, al), bb, acc[b], 0, 0, 0);
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, am), bb, acc[b], 0, 0, 0);
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, ah), bb, acc[b], 0, 0, 0);
+        for (int b = 0; b < 8; ++b)
+          c[e][b] = static_cast<float>(kInt4 ? static_cast<int>(w[st][4 * grp + e][0] << (28 - 4 * b)) >> 28
+                                             : static_cast<int>(w[st][4 * grp + e][b >> 2] << (24 - 8 * (b & 3))) >> 24);
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        u32x2_t bv;
+        bv[0] = pack2<bf16_t>(c[0][b], c[1][b]);
+        bv[1] = pack2<bf16_t>(c[2][b], c[3][b]);
+        const short4_t bb = __builtin_bit_cast(short4_t, bv);
+        // smallest piece first
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, al), bb, acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, am), bb, acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, ah), bb, acc[b], 0, 0, 0);
+      }
     }
   };
   auto multiply = [&](int st) {
@@ -338,7 +348,8 @@ int launch_vec(const DxArgs &a, dim3 grid, size_t lds, hipStream_t s)
 {
   // one vector load per stage for the gradient when its four values are neighbours and the vector is aligned;
   // with residue classes the workgroup's piece of dY goes through LDS when it fits where the partial tiles go later
-  const bool vec = a.V == 1 && a.N % 4 == 0 && a.N >= 4 && aligned_to(a.dy, 4 * sizeof(XT));
+  const size_t vbytes = kDxIter * sizeof(XT) > 16 ? 16 : kDxIter * sizeof(XT);
+  const bool vec = a.V == 1 && a.N % kDxIter == 0 && a.N >= kDxIter && aligned_to(a.dy, vbytes);
   if (vec) {
     hipLaunchKernelGGL((dxrows_kernel<XT, CT, kInt4, GRAD_VECTOR>), grid, dim3(kDxThreads), lds, s, a);
     return launch_status();
