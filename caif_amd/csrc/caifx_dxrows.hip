@@ -84,7 +84,18 @@ __global__ __launch_bounds__(kDxThreads) void dxrows_kernel(DxArgs a)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int j = lane & 15;
   const int q = lane >> 4;
-  const int64_t k0 = static_cast<int64_t>(blockIdx.x) * kDxSlab;
+  // Packed int4: a slab's 128 columns are half a cache line of every weight row, and the other half belongs to the
+  // neighbouring slab.  Workgroups go to the 8 XCDs (each with its own L2) in turn by their linear id, so neighbours
+  // would fetch every line into two L2s; slabs 2p and 2p + 1 are therefore given to workgroups 8 apart (the same
+  // XCD, dispatched together), in blocks of 16 slabs, when the grid's width keeps that pairing (a multiple of 8).
+  int slab = blockIdx.x;
+  if constexpr (kInt4) {
+    if ((gridDim.x & 7) == 0 && slab < static_cast<int>(gridDim.x & ~15u)) {
+      const int t = slab >> 4, h = (slab >> 3) & 1, x = slab & 7;
+      slab = 16 * t + 2 * x + h;
+    }
+  }
+  const int64_t k0 = static_cast<int64_t>(slab) * kDxSlab;
   const int cls = blockIdx.y / a.ranges;
   const int64_t rows_class = (a.N - cls + a.V - 1) / a.V;              // rows n = cls + V*i, i < rows_class
   const int64_t n_lo = static_cast<int64_t>(blockIdx.y - cls * a.ranges) * a.rows_per_wg;      // (i, not n, from here on)
