@@ -1,7 +1,6 @@
 // extern "C" entry points of the dequant-GEMM seam: argument validation and kernel choice.
 #include "caifx_internal.hpp"
 
-#include <cstdlib>
 
 #include <atomic>
 
@@ -277,10 +276,7 @@ static int backward_impl(int64_t M, int64_t N, int64_t K, const void *dy, int dy
   // up to 16 rows of int8 codes (scale vectors through residue classes of the rows, one scale, none) or of int4
   // codes in groups of 128 or more: one pass over the weight, whatever the compute type (16-bit compute types on
   // the 16-bit matrix cores)
-  bool few_rows_first = M <= 16 && (w_kind == CAIFX_W_INT8 || w_kind == CAIFX_W_INT4_GROUP);
-#ifdef CAIFX_DEV
-  if (const char *e = getenv("CAIFX_DX_FEW")) few_rows_first = e[0] == '1' && M <= 16;
-#endif
+  const bool few_rows_first = M <= 16 && (w_kind == CAIFX_W_INT8 || w_kind == CAIFX_W_INT4_GROUP);
   if (few_rows_first) {
     st = dxrows_backward(a, s);
     if (st != CAIFX_ERR_UNSUPPORTED) return finish_add(st, addend, dx, dx_dtype, M * K, stream);

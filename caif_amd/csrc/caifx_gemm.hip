@@ -3,7 +3,6 @@
 #include "caifx_gemm_regw.hpp"
 #include "caifx_gemm_tile.hpp"
 
-#include <cstdlib>
 
 namespace caifx {
 namespace {
@@ -84,13 +83,6 @@ SplitPlan plan_split(int64_t M, int64_t C, int64_t R, bool grouped)
   // one workgroup per compute unit: two resident 128-row workgroups run about as fast as one after the other, so
   // parts beyond 256 workgroups only add partial tiles (224 tiles in 2 parts measured 90 us against 75 us unsplit)
   int64_t target = 256, most = 8, least = 8;
-#ifdef CAIFX_DEV
-  if (M <= 32) {
-    if (const char *e = getenv("CAIFX_SPLIT_TARGET")) target = atoi(e);
-    if (const char *e = getenv("CAIFX_SPLIT_MOST")) most = atoi(e);
-    if (const char *e = getenv("CAIFX_SPLIT_LEAST")) least = atoi(e);
-  }
-#endif
   int64_t k = target / tiles;
   if (k > most) k = most;
   if (k > steps / least) k = steps / least;

@@ -32,7 +32,6 @@
 #include "caifx_gemm_regw.hpp"
 
 #include <atomic>
-#include <cstdlib>
 #include <type_traits>
 
 namespace caifx {
@@ -377,10 +376,6 @@ int mfma_regw_forward(const GemmArgs &a, hipStream_t s)
 
 int mfma_forward(const GemmArgs &a, hipStream_t s)
 {
-#ifdef CAIFX_DEV
-  if (const char *sw = getenv("CAIFX_REGW"))
-    if (sw[0] == '0') return mfma_tiled_forward(a, s);
-#endif
   int st = mfma_regw_forward(a, s);
   if (st == CAIFX_ERR_UNSUPPORTED) st = mfma_regw8_forward(a, s);
   return st == CAIFX_ERR_UNSUPPORTED ? mfma_tiled_forward(a, s) : st;

@@ -25,7 +25,6 @@
 #include "caifx_gemm_regw.hpp"
 
 #include <atomic>
-#include <cstdlib>
 #include <type_traits>
 
 namespace caifx {
@@ -470,10 +469,6 @@ template <typename CT, bool kGrouped> int launch(const Regw8Args &t, int64_t row
 
 int mfma_regw8_forward(const GemmArgs &a, hipStream_t s)
 {
-#ifdef CAIFX_DEV
-  if (const char *sw = getenv("CAIFX_REGW8"))
-    if (sw[0] == '0') return CAIFX_ERR_UNSUPPORTED;
-#endif
   const bool grouped = a.offsets != nullptr;
   if (a.w.kind != CAIFX_W_INT8) return CAIFX_ERR_UNSUPPORTED;
   if (a.epilogue != 0) {
