@@ -203,10 +203,12 @@ __device__ __forceinline__ uint32_t quantize_int8_x4(const floatx4_t &v, const f
 
 // One scale for the whole tensor, 16 consecutive elements per thread (16-byte aligned input and output,
 // n % 16 == 0): same arithmetic per element as quantize_int8_kernel, the reciprocal taken once per thread.
+// The blocks walk the tensor from its end: the maximum pass before this one read it front to back, so its tail
+// is what the memory-side cache still holds.
 __global__ void quantize_int8_tensor_x16_kernel(const float *__restrict__ in, int8_t *__restrict__ out,
                                                 const float *__restrict__ scale, int64_t n16)
 {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t i = static_cast<int64_t>(gridDim.x - 1 - blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= n16) return;
   const float s = scale[0];
   const float one = (s > 0.0f) ? 1.0f / s : 0.0f;
