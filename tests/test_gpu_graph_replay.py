@@ -102,3 +102,57 @@ def test_replays_equal_eager_results():
         for k in want:
             assert torch.equal(got[k], want[k]), (rep, k)
     assert not np.isnan(got["comb"].float().cpu().numpy()).any()
+
+
+def test_replays_of_the_large_forward_kernels_and_the_few_row_gradient():
+    # the int4 and int8 forward kernels that keep the weight out of the shared operand tiles (first launched inside
+    # the capture: they raise their LDS limit there), the grouped int8 form, and the few-row input gradient with its
+    # gradient piece staged through LDS (three residue classes) and its adding pass
+    dev = torch.device("cuda")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+
+    def int8(n, k):
+        q, s = T.quantize_int8(torch.empty(k, n, device=dev).normal_(0, 0.02, generator=gen), per_channel=True)
+        return T.FrozenWeight(q.reshape(-1), T.W_INT8, s, n, k, n)
+
+    N, K, M = 2048, 640, 4096
+    fw8 = int8(N, K)
+    p4, s4 = T.quantize_int4_per_group(torch.empty(N, 512, device=dev).normal_(0, 0.02, generator=gen), 128)
+    fw4 = T.FrozenWeight(p4, T.W_INT4_GROUP, s4, N, 512, 1, 128)
+    E, rows = 8, 16384
+    gw = T.GroupedFrozenWeights([int8(512, 256) for _ in range(E)])
+    offsets = torch.tensor([0, 2000, 2000, 4100, 6148, 9000, 12000, 15000, rows], dtype=torch.int32, device=dev)
+    fwd = int8(1536, 1024)                                           # K mod N = 1024: three residue classes of rows
+    x8 = torch.empty(M, K, device=dev, dtype=torch.bfloat16)
+    x4 = torch.empty(M, 512, device=dev, dtype=torch.bfloat16)
+    xg = torch.empty(rows, 256, device=dev, dtype=torch.bfloat16)
+    dy = torch.empty(16, 1536, device=dev, dtype=torch.bfloat16)
+    ws = torch.empty(1 << 22, dtype=torch.uint8, device=dev)
+
+    def refill():
+        for t, std in ((x8, 1.0), (x4, 1.0), (xg, 1.0), (dy, 1e-2)):
+            t.copy_(torch.empty(t.shape, device=dev).normal_(0, std, generator=gen))
+
+    def run():
+        return (T.qlinear_forward(x8, fw8, T.BF16, T.BF16), T.qlinear_forward(x4, fw4, T.BF16, T.F32),
+                T.qlinear_grouped_forward(xg, offsets, gw, T.BF16, T.BF16),
+                T.qlinear_backward_input(dy, fwd, T.BF16, T.F32, workspace=ws))
+
+    refill()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            outs = run()
+    torch.cuda.synchronize()
+    for rep in range(3):
+        refill()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        want = run()
+        torch.cuda.synchronize()
+        for got, ref in zip(outs, want):
+            assert torch.equal(got, ref), rep
