@@ -123,6 +123,110 @@ __device__ __forceinline__ void segment_rows(const int32_t *offsets, int e, int6
   hi = hi < lo ? lo : (hi > m ? m : hi);
 }
 
+// Which tile of a grouped launch a workgroup owns.  Row tiles of BM rows are counted over all experts, expert by
+// expert, and crossed with col_tiles column tiles, column tile last; XCD x (workgroup id mod 8, each XCD has its own
+// L2) takes the x-th contiguous eighth of that list, so one expert's weight and one row tile's activations are
+// fetched into one L2.  Every wave works the numbering out on its own: lane l takes expert base + l and a scan
+// over the lanes gives the running tile count.  A tile starts with this search, and each dependent global load in
+// it is a memory round trip during which the compute unit's share of the tile does nothing: with up to 64 experts
+// every lane asks for its expert's offsets and pointers in one go, before the tile is known, and the owner's
+// values are then read from its lane; with more, the offsets are walked twice and the pointers fetched last.
+// False: the workgroup has no tile (the grid is an upper bound).  pos: the tile's index in the list.
+struct GroupedTile {
+  int e;                   // expert
+  int64_t row0, row_end;   // first row of the tile, end of the expert's segment
+  int64_t col_tile;
+  int64_t pos;
+  const void *wq;
+  const void *scales;      // null when scales_ptrs is
+};
+template <int BM>
+__device__ __forceinline__ bool grouped_tile(const int32_t *offsets, int num_experts, int64_t M, int64_t col_tiles,
+                                             const void *const *wq_ptrs, const void *const *scales_ptrs, int lane,
+                                             GroupedTile &out)
+{
+  if (num_experts <= 64) {
+    int my_lo = 0, my_hi = 0;
+    uint64_t my_w = 0, my_s = 0;
+    if (lane < num_experts) {
+      segment_rows(offsets, lane, M, my_lo, my_hi);
+      my_w = reinterpret_cast<uint64_t>(wq_ptrs[lane]);
+      if (scales_ptrs) my_s = reinterpret_cast<uint64_t>(scales_ptrs[lane]);
+    }
+    const int tiles = (my_hi - my_lo + BM - 1) / BM;
+    int incl = tiles;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+    const int64_t total = static_cast<int64_t>(__shfl(incl, 63, 64)) * col_tiles;
+    const int64_t per_xcd = (total + 7) >> 3;
+    const int64_t slot = blockIdx.x >> 3;
+    const int64_t pos = static_cast<int64_t>(blockIdx.x & 7) * per_xcd + slot;
+    if (slot >= per_xcd || pos >= total) return false;
+    const int t = static_cast<int>(pos / col_tiles);
+    const unsigned long long owners = __ballot(incl > t);
+    if (owners == 0) return false;
+    const int src = __builtin_ctzll(owners);
+    out.e = src;
+    out.pos = pos;
+    out.col_tile = pos - static_cast<int64_t>(t) * col_tiles;
+    out.row0 = __shfl(my_lo, src, 64) + static_cast<int64_t>(t - __shfl(incl - tiles, src, 64)) * BM;
+    out.row_end = __shfl(my_hi, src, 64);
+    const uint32_t wl = __shfl(static_cast<uint32_t>(my_w), src, 64), wh = __shfl(static_cast<uint32_t>(my_w >> 32), src, 64);
+    const uint32_t sl = __shfl(static_cast<uint32_t>(my_s), src, 64), sh = __shfl(static_cast<uint32_t>(my_s >> 32), src, 64);
+    out.wq = reinterpret_cast<const void *>((static_cast<uint64_t>(wh) << 32) | wl);
+    out.scales = reinterpret_cast<const void *>((static_cast<uint64_t>(sh) << 32) | sl);
+    return true;
+  }
+  int total_rt = 0;
+  for (int base = 0; base < num_experts; base += 64) {
+    const int my = base + lane;
+    int tiles = 0;
+    if (my < num_experts) {
+      int slo, shi;
+      segment_rows(offsets, my, M, slo, shi);
+      tiles = (shi - slo + BM - 1) / BM;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) tiles += __shfl_xor(tiles, o, 64);
+    total_rt += tiles;
+  }
+  const int64_t total = static_cast<int64_t>(total_rt) * col_tiles;
+  const int64_t per_xcd = (total + 7) >> 3;
+  const int64_t slot = blockIdx.x >> 3;
+  const int64_t pos = static_cast<int64_t>(blockIdx.x & 7) * per_xcd + slot;
+  if (slot >= per_xcd || pos >= total) return false;
+  int t = static_cast<int>(pos / col_tiles);
+  out.pos = pos;
+  out.col_tile = pos - static_cast<int64_t>(t) * col_tiles;
+  for (int base = 0; base < num_experts; base += 64) {
+    const int my = base + lane;
+    int my_lo = 0, my_hi = 0;
+    if (my < num_experts) segment_rows(offsets, my, M, my_lo, my_hi);
+    const int tiles = (my_hi - my_lo + BM - 1) / BM;
+    int incl = tiles;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+    const unsigned long long owners = __ballot(incl > t);
+    if (owners != 0) {
+      const int src = __builtin_ctzll(owners);
+      out.e = base + src;
+      out.row0 = __shfl(my_lo, src, 64) + static_cast<int64_t>(t - __shfl(incl - tiles, src, 64)) * BM;
+      out.row_end = __shfl(my_hi, src, 64);
+      out.wq = wq_ptrs[out.e];
+      out.scales = scales_ptrs ? scales_ptrs[out.e] : nullptr;
+      return true;
+    }
+    t -= __shfl(incl, 63, 64);
+  }
+  return false;
+}
+
 // v_mfma_f32_32x32x16 in the 16-bit compute type CT: A is 32 rows x 16 (lane l supplies row l % 32, reduction
 // elements 8 * (l / 32) .. + 7), B likewise by column; of the 32 x 32 result lane l holds column l % 32 and, in
 // register r, row 8 * (r / 4) + 4 * (l / 32) + r % 4.

@@ -91,57 +91,15 @@ __global__ __launch_bounds__(512, 2) void qgemm_regw8_kernel(Regw8Args g)
   int64_t stamp_pos = -1;
   const int64_t col_tiles = (g.N + kBN - 1) / kBN;
   if constexpr (kGrouped) {
-    int total_rt = 0;
-    for (int base = 0; base < g.num_experts; base += 64) {
-      const int my = base + lane;
-      int tiles = 0;
-      if (my < g.num_experts) {
-        int slo, shi;
-        segment_rows(g.offsets, my, g.M, slo, shi);
-        tiles = (shi - slo + BM - 1) / BM;
-      }
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) tiles += __shfl_xor(tiles, o, 64);
-      total_rt += tiles;
-    }
-    const int64_t total = static_cast<int64_t>(total_rt) * col_tiles;
-    const int64_t per_xcd = (total + 7) >> 3;
-    const int64_t slot = blockIdx.x >> 3;
-    const int64_t pos = static_cast<int64_t>(blockIdx.x & 7) * per_xcd + slot;
-    if (slot >= per_xcd || pos >= total) return;
-    int t = static_cast<int>(pos / col_tiles);
-    col0 = (pos - static_cast<int64_t>(t) * col_tiles) * kBN;
-    int e = 0;
-    int64_t lo = 0, hi = 0;
-    bool found = false;
-    for (int base = 0; base < g.num_experts && !found; base += 64) {
-      const int my = base + lane;
-      int my_lo = 0, my_hi = 0;
-      if (my < g.num_experts) segment_rows(g.offsets, my, g.M, my_lo, my_hi);
-      const int tiles = (my_hi - my_lo + BM - 1) / BM;
-      int incl = tiles;
-#pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        const int up = __shfl_up(incl, o, 64);
-        if (lane >= o) incl += up;
-      }
-      const unsigned long long owners = __ballot(incl > t);
-      if (owners != 0) {
-        const int src = __builtin_ctzll(owners);
-        e = base + src;
-        t -= __shfl(incl - tiles, src, 64);
-        lo = __shfl(my_lo, src, 64);
-        hi = __shfl(my_hi, src, 64);
-        found = true;
-      } else {
-        t -= __shfl(incl, 63, 64);
-      }
-    }
-    if (!found) return;
-    row0 = lo + static_cast<int64_t>(t) * BM;
-    row_end = hi;
-    wq = static_cast<const uint8_t *>(g.wq_ptrs[e]);
-    scales = g.scales_ptrs ? static_cast<const float *>(g.scales_ptrs[e]) : nullptr;
+    GroupedTile gt;
+    if (!grouped_tile<BM>(g.offsets, g.num_experts, g.M, col_tiles, g.wq_ptrs, g.scales_ptrs, lane, gt)) return;
+    const int e = gt.e;
+    const int64_t pos = gt.pos;
+    col0 = gt.col_tile * kBN;
+    row0 = gt.row0;
+    row_end = gt.row_end;
+    wq = static_cast<const uint8_t *>(gt.wq);
+    scales = static_cast<const float *>(gt.scales);
     if (g.stamps && threadIdx.x == 0 && pos < g.stamps_capacity) {
       const int64_t rows = row_end - row0 < BM ? row_end - row0 : BM;
       g.stamps[4 * pos] = static_cast<unsigned long long>(e);

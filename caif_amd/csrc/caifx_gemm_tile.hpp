@@ -129,65 +129,18 @@ __global__ __launch_bounds__(2 * kCW * 64, (kCW == 8 || (BM == 128 && (kW == W_C
   const uint8_t *wq = static_cast<const uint8_t *>(g.wq);
   const void *scales = g.scales;
   if constexpr (kGrouped) {
-    // Row tiles are counted over all experts.  Every wave works the numbering out on its own: lane l
-    // takes expert base+l and an inclusive scan over the lanes gives the running tile count.
-    // Workgroups are handed to the 8 XCDs in turn (linear id mod 8) and each XCD has its own L2, so
-    // the tiles are numbered expert by expert, row tile by row tile, column tile last, and XCD x
-    // takes the x-th contiguous eighth of that list: one expert's weights (and one row tile's
-    // activations) are then fetched into one L2 instead of all eight.  The grid is an upper bound
-    // padded to a multiple of 8; the exact number of tiles comes from the offsets.
+    // tiles are numbered expert by expert, row tile by row tile, column tile last, one contiguous eighth of the
+    // list per XCD (grouped_tile); the grid is an upper bound padded to a multiple of 8
     const int64_t col_tiles = (C + BC - 1) / BC;
-    int total_rt = 0;
-    for (int base = 0; base < g.num_experts; base += 64) {
-      const int my = base + lane;
-      int tiles = 0;
-      if (my < g.num_experts) {
-        int slo, shi;
-        segment_rows(g.offsets, my, g.M, slo, shi);
-        tiles = (shi - slo + BM - 1) / BM;
-      }
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) tiles += __shfl_xor(tiles, o, 64);
-      total_rt += tiles;
-    }
-    const int64_t total = static_cast<int64_t>(total_rt) * col_tiles;
-    const int64_t per_xcd = (total + 7) >> 3;
-    const int64_t slot = blockIdx.x >> 3;
-    const int64_t pos = static_cast<int64_t>(blockIdx.x & 7) * per_xcd + slot;
-    if (slot >= per_xcd || pos >= total) return;
-    int t = static_cast<int>(pos / col_tiles);
-    col_tile = pos - static_cast<int64_t>(t) * col_tiles;
-    int e = 0;
-    int64_t lo = 0, hi = 0;
-    bool found = false;
-    for (int base = 0; base < g.num_experts && !found; base += 64) {
-      const int my = base + lane;
-      int my_lo = 0, my_hi = 0;
-      if (my < g.num_experts) segment_rows(g.offsets, my, g.M, my_lo, my_hi);
-      const int tiles = (my_hi - my_lo + BM - 1) / BM;
-      int incl = tiles;
-#pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        const int up = __shfl_up(incl, o, 64);
-        if (lane >= o) incl += up;
-      }
-      const unsigned long long owners = __ballot(incl > t);
-      if (owners != 0) {
-        const int src = __builtin_ctzll(owners);
-        e = base + src;
-        t -= __shfl(incl - tiles, src, 64);
-        lo = __shfl(my_lo, src, 64);
-        hi = __shfl(my_hi, src, 64);
-        found = true;
-      } else {
-        t -= __shfl(incl, 63, 64);
-      }
-    }
-    if (!found) return;
-    row_lo = lo + static_cast<int64_t>(t) * BM;
-    row_hi = hi;
-    wq = static_cast<const uint8_t *>(g.wq_ptrs[e]);
-    scales = g.scales_ptrs ? g.scales_ptrs[e] : nullptr;
+    GroupedTile gt;
+    if (!grouped_tile<BM>(g.offsets, g.num_experts, g.M, col_tiles, g.wq_ptrs, g.scales_ptrs, lane, gt)) return;
+    const int e = gt.e;
+    const int64_t pos = gt.pos;
+    col_tile = gt.col_tile;
+    row_lo = gt.row0;
+    row_hi = gt.row_end;
+    wq = static_cast<const uint8_t *>(gt.wq);
+    scales = gt.scales;
     if (g.stamps && threadIdx.x == 0 && pos < g.stamps_capacity) {
       const int64_t rows = row_hi - row_lo < BM ? row_hi - row_lo : BM;
       g.stamps[4 * pos] = static_cast<unsigned long long>(e);
