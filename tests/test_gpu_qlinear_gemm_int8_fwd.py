@@ -133,3 +133,24 @@ def test_grouped_segments(orc, kind, N, K):
         err = max_rel_err(y[sel], orc.frozen_linear_forward(xh[sel], pairs[e][0], 2))
         assert err <= TOL and err <= TIGHT, (kind, e, err)
     assert (y[total:] == 7.0).all()
+
+
+def test_grouped_more_than_64_experts(orc):
+    # the tile search takes the offsets 64 experts at a time: segments on both sides of that edge, empty ones included
+    rng = np.random.default_rng(70)
+    N, K = 512, 256
+    counts = rng.integers(60, 260, 70)
+    counts[[0, 62, 63, 64, 65, 69]] = [0, 129, 0, 7, 300, 33]
+    E = len(counts)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    total = int(offsets[-1])
+    pairs = [make_weight(orc, rng, N, K, "int8pc") for _ in range(E)]
+    gw = T.GroupedFrozenWeights([p[1] for p in pairs])
+    x = dev_as(rng.normal(0, 1, (total, K)), 2)
+    y = host(T.qlinear_grouped_forward(x, dev(offsets), gw, 2))
+    xh = host(x)
+    for e in (1, 61, 62, 64, 65, 68, 69):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        sel = np.unique(np.concatenate([rng.choice(hi - lo, min(8, hi - lo), replace=False), [0, hi - lo - 1]])) + lo
+        err = max_rel_err(y[sel], orc.frozen_linear_forward(xh[sel], pairs[e][0], 2))
+        assert err <= TOL and err <= TIGHT, (e, err)
