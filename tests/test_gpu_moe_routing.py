@@ -19,7 +19,9 @@ def _case(rng, Tk, top_k, E, bad=0):
 
 
 @pytest.mark.parametrize("Tk,top_k,E,cap", [(1, 1, 1, 0), (37, 3, 5, 0), (300, 6, 64, 0), (257, 2, 70, 0),
-                                            (128, 4, 8, 9), (64, 1, 3, 5), (4096, 6, 64, 0), (1000, 8, 130, 40)])
+                                            (128, 4, 8, 9), (64, 1, 3, 5), (4096, 6, 64, 0), (1000, 8, 130, 40),
+                                            # past what one workgroup's LDS holds: the launches over a workspace
+                                            (16384, 8, 64, 0), (3000, 6, 200, 50), (9000, 4, 64, 500)])
 def test_dispatch_map_matches_reference_order(orc, Tk, top_k, E, cap):
     rng = np.random.default_rng(Tk + top_k + E)
     idx = _case(rng, Tk, top_k, E, bad=3 if Tk > 10 else 0)
